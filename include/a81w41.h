@@ -89,11 +89,21 @@ int a81w41_gemv_repack_A81W41_fp16(const void *A_repack_dev, const void *B_repac
  * quantized_gemx_kernels.cc:349-582): C[M][N] row-major from 80 B activation
  * blocks and the 384 B weight blob.  Any M >= 1 (rows past M are never read).
  * Calls with M > 8 may split the K range of some tiles and park partial tiles in a
- * per-device scratch (64 MiB, allocated by a81w41_context_create or on the first
- * such call, kept until the process ends): launches of this function on one device
- * must not overlap in time.  Results do not depend on timing. */
+ * scratch (64 MiB) that belongs to `stream`: it is allocated by the first such call on
+ * that stream (which therefore cannot be captured into a graph; later calls can) and kept
+ * until the process ends, at most 16 streams per device.  Calls on one stream are ordered
+ * by the stream, calls on different streams use different scratches, so no two launches
+ * ever share partial tiles.  Results do not depend on timing. */
 int a81w41_gemm_repack_A81W41_fp32(const void *A_repack_dev, const void *B_repack_dev, float *C_dev,
                                    int M, int N, int K, void *stream);
+
+/* Test hook, host only (no device is touched): walks the work list the M > 8 kernels would be
+ * launched with for an M x N x K call on a device that holds `resident_workgroups` of them on
+ * `cus` compute units (tile = 2: 64 x 64 tiles, 1: 32 x 128 tiles).  Returns the number of
+ * partial tiles the K split parks (>= 0) if every tile and every K chunk is covered exactly
+ * once, the tile numbering is one-to-one and no two chunks share a partial tile; a negative
+ * code names the violated property. */
+int a81w41_gemm_schedule_selfcheck(int M, int N, int K, int resident_workgroups, int cus, int tile);
 
 /* The int32 block dots both kernels form before scaling (iacc_low / iacc_high,
  * quantized_gemx_kernels.cc:161-168 and :430-457), exposed for parity checks:
@@ -129,7 +139,7 @@ int a81w41_gemv_repack_A80W40(const void *A_repack_dev, const void *B_repack_dev
  * (the reference's 2 x 2 blocking reads past the blob when N/8 is odd; this does not).
  * Both operands are first rewritten into `workspace_dev` in the 80 B / 384 B form of the
  * A81W41 contraction (min = -8 d_w, scaled sum = d_a * sum(q), both exact), which then runs
- * on the matrix cores; the same scratch rule as a81w41_gemm_repack_A81W41_fp32 applies.
+ * on the matrix cores; the same per-stream scratch as a81w41_gemm_repack_A81W41_fp32's is used.
  * The workspace is the caller's: 16-byte aligned, at least ..._workspace_bytes(M, N, K). */
 size_t a81w41_gemm_repack_A80W40_workspace_bytes(int M, int N, int K);
 int a81w41_gemm_repack_A80W40(const void *A_repack_dev, const void *B_repack_dev, float *C_dev,
@@ -144,8 +154,9 @@ int a81w41_block_idot_A80W40(const void *A_repack_dev, const void *B_repack_dev,
  * a81w41_context replaces ModelContext (QwenOperator.h:34-43): it owns the
  * device scratch every layer quantises its activations into, sized for
  * max_rows x max_cols activations (the reference sizes it for 4096 x 12288,
- * QwenForCausalLM.cc:101-113).  Like the reference's, it is shared by all
- * layers, so forward calls on one context must not overlap. */
+ * QwenForCausalLM.cc:101-113), and the 64 MiB of partial tiles its layers' M > 8 calls
+ * may park.  Like the reference's, it is shared by all its layers, so forward calls on
+ * one context must not overlap; calls on different contexts may. */
 typedef struct a81w41_context a81w41_context;
 typedef struct a81w41_linear a81w41_linear;
 
@@ -240,6 +251,17 @@ int a81w41_qwen3_set_linear_blobs(a81w41_qwen3 *model, int layer, int which, con
 int a81w41_qwen3_set_norm(a81w41_qwen3 *model, int layer, int which, const float *weight);
 /* Embedding table [vocab][hidden] as IEEE binary16 bit patterns, host. */
 int a81w41_qwen3_set_embedding(a81w41_qwen3 *model, const uint16_t *table_fp16);
+/* Test switches: each keeps one fusion of the one-token / prefill pass off, so that the fused
+ * pass can be compared with the separate kernels, or fixes the attention's key split.  The
+ * results of a pass do not change by a bit with UNFUSED, ATTN_FP32 and NO_PAIR. */
+enum {
+    A81W41_QWEN3_OPT_UNFUSED = 0,          /* separate elementwise kernels and quantiser launches */
+    A81W41_QWEN3_OPT_ATTN_FP32 = 1,        /* one-token attention writes fp32, o_proj quantises it */
+    A81W41_QWEN3_OPT_NO_PAIR = 2,          /* gate_up writes fp32, down_proj's prologue does SiLU*mul */
+    A81W41_QWEN3_OPT_VECTOR_ATTENTION = 3, /* prefill attention on the vector kernel */
+    A81W41_QWEN3_OPT_ATTENTION_SPLIT = 4   /* value 1..16: shares per head of the one-token attention; 0: automatic */
+};
+int a81w41_qwen3_set_option(a81w41_qwen3 *model, int option, int value);
 /* Forget the cached context (position 0). */
 int a81w41_qwen3_reset(a81w41_qwen3 *model);
 /* Qwen3ForCausalLM::forward: n_tokens new token ids (host) on top of the cached context;

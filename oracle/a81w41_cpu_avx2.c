@@ -6,9 +6,11 @@
  * 6-row M tile (quantized_gemx_kernels.cc:129-193, :364-582) and the serial
  * quantizer (:693-911).  Every lane performs the same IEEE operations in the
  * same order as the scalar oracle, so the two agree bit for bit (checked in
- * tests/test_oracle_avx2.py).  Integer dots use maddubs+madd, the reference's
- * plain-AVX2 branch (lib.h:50-53); the products cannot saturate here
- * (2*15*127 < 32767).
+ * tests/test_oracle_avx2.py).  Integer dots follow mul_sum_us8_pairs_acc_int32x8
+ * (lib.h:45-55), whose branch is picked by the compiler flags: dpbusd with
+ * AVX512-VNNI + VL or with AVX-VNNI, else maddubs+madd (the products cannot
+ * saturate there: 2*15*127 < 32767).  The Makefile builds one library per
+ * branch from this file; oracle/ora.py loads the best one the host CPU runs.
  */
 #include <immintrin.h>
 #include <omp.h>
@@ -20,7 +22,24 @@
 int avx_max_threads(void) { return omp_get_max_threads(); }
 
 static inline __m256i dot_u8s8_acc(__m256i acc, __m256i u, __m256i s) {
+#if defined(__AVX512VNNI__) && defined(__AVX512VL__)
+    return _mm256_dpbusd_epi32(acc, u, s);
+#elif defined(__AVXVNNI__)
+    return _mm256_dpbusd_avx_epi32(acc, u, s);
+#else
     return _mm256_add_epi32(acc, _mm256_madd_epi16(_mm256_maddubs_epi16(u, s), _mm256_set1_epi16(1)));
+#endif
+}
+
+/* Which branch of lib.h:45-55 this build of the file takes. */
+const char *avx_dot_branch(void) {
+#if defined(__AVX512VNNI__) && defined(__AVX512VL__)
+    return "avx512-vnni dpbusd";
+#elif defined(__AVXVNNI__)
+    return "avx-vnni dpbusd";
+#else
+    return "avx2 maddubs+madd";
+#endif
 }
 
 static inline int hsum_i32(__m256i v) {

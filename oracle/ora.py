@@ -13,7 +13,6 @@ import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB = os.path.join(_HERE, "liba81w41_oracle.so")
-_AVX = os.path.join(_HERE, "liba81w41_cpu_avx2.so")
 
 
 def build(force: bool = False) -> None:
@@ -186,10 +185,51 @@ def quantize_weight_q40(w: np.ndarray):
 
 # ------------------------------------------------------------------ AVX2 + OpenMP port (timed CPU baseline)
 
-def avx():
+AVX_BRANCHES = {  # integer-dot branch of the reference's lib.h:45-55 -> (library, /proc/cpuinfo flags it needs)
+    "avx512vnni": ("liba81w41_cpu_avx512vnni.so", {"avx512_vnni", "avx512vl", "avx512f", "avx2", "fma", "f16c"}),
+    "avxvnni": ("liba81w41_cpu_avxvnni.so", {"avx_vnni", "avx2", "fma", "f16c"}),
+    "avx2": ("liba81w41_cpu_avx2.so", {"avx2", "fma", "f16c"}),
+}
+_avx_libs = {}
+
+
+def cpu_flags():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("flags"):
+                    return set(line.split(":", 1)[1].split())
+    except OSError:
+        pass
+    return set()
+
+
+def avx_branches_supported():
+    """Branches this host's CPU can run, best first (the order the reference's #if chain prefers)."""
+    flags = cpu_flags()
+    return [b for b, (_, need) in AVX_BRANCHES.items() if need <= flags]
+
+
+def avx(branch=None):
+    """The AVX2+OpenMP port; ``branch`` None = the best integer-dot branch this CPU supports."""
     global _avx
-    if _avx is None:
-        L = _load(_AVX)
+    if branch is None:
+        if _avx is not None:
+            return _avx
+        sup = avx_branches_supported()
+        if not sup:
+            raise OSError("this CPU lacks AVX2/FMA/F16C: the CPU-baseline port cannot run here")
+        _avx = avx(sup[0])
+        return _avx
+    if branch not in _avx_libs:
+        L = _load(os.path.join(_HERE, AVX_BRANCHES[branch][0]))
+        L.avx_dot_branch.restype = C.c_char_p
+        _avx_libs[branch] = _bind_avx(L)
+    return _avx_libs[branch]
+
+
+def _bind_avx(L):
+    if True:
         for name in ("avx_quantize_row_q8_1_repack_fp16", "avx_quantize_row_q8_1_repack_fp32"):
             getattr(L, name).argtypes = [_vp, _vp, _i64]
             getattr(L, name).restype = None
@@ -197,5 +237,4 @@ def avx():
             getattr(L, name).argtypes = [_vp, _vp, _vp, _i, _i, _i, _i]
             getattr(L, name).restype = None
         L.avx_max_threads.restype = _i
-        _avx = L
-    return _avx
+    return L

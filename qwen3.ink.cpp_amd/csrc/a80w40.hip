@@ -76,7 +76,7 @@ size_t gemm_a80w40_workspace_bytes(int M, int N, int K) {
 }
 
 hipError_t launch_gemm_a80w40(const void* A, const void* B, float* C, int M, int N, int K, void* workspace,
-                              hipStream_t s) {
+                              const GemmScratch& ws, hipStream_t s) {
     const size_t nb_k = (size_t)K / 64;
     uint8_t* a32 = static_cast<uint8_t*>(workspace);
     uint8_t* b32 = a32 + round_up_256((size_t)M * nb_k * kABlock32);
@@ -87,7 +87,7 @@ hipError_t launch_gemm_a80w40(const void* A, const void* B, float* C, int M, int
     hipLaunchKernelGGL(w80_to_w81_fp32_kernel, dim3((unsigned)((b_chunks + 255) / 256)), dim3(256), 0, s,
                        static_cast<const uint8_t*>(B), reinterpret_cast<uint4*>(b32), b_chunks);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
-    return launch_gemm_fp32(a32, b32, C, M, N, K, s);
+    return launch_gemm_fp32(a32, b32, C, M, N, K, ws, s);
 }
 
 }  // namespace a81w41

@@ -3,8 +3,24 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 namespace a81w41 {
+
+// Environment overrides of the kernel selection exist in tuning builds only (make TUNING=1); the
+// default build never reads the environment.
+inline const char* tuning_env(const char* name) {
+#ifdef A81W41_TUNING
+    return getenv(name);
+#else
+    (void)name;
+    return nullptr;
+#endif
+}
+inline int tuning_env_int(const char* name) {
+    const char* v = tuning_env(name);
+    return v ? atoi(v) : 0;
+}
 
 constexpr int kWBlock16 = 320;  // q4_repack_2x8_fp16
 constexpr int kWBlock32 = 384;  // q4_repack_2x8_fp32
@@ -45,14 +61,29 @@ hipError_t launch_gemv_add_norm(const float* x, const GemvPrologue& pro, void* a
 // add_norm in front, and behind it, instead of the N = 2 I outputs of a gate|up matrix (gate rows, then
 // up rows), the quantised 72 B blocks of silu(gate) * up in pro.pair_out: the next linear's input, to
 // be contracted with launch_gemv_fp16.  I % 32 == 0; needs gemv_add_norm_fits(K).
+bool gemv_pair_fits(int N, int K);
 hipError_t launch_gemv_add_norm_silu_pair(const float* x, const GemvPrologue& pro, const void* B_gate_up, int N, int K,
                                           hipStream_t s);
-hipError_t launch_gemm_fp32(const void* A, const void* B, float* C, int M, int N, int K, hipStream_t s);
-// Allocates the per-device scratch of the GEMM (partial tiles of its K-split path) if it does not
-// exist yet.  launch_gemm_fp32 does the same on first use; doing it up front keeps that first
-// use legal inside a stream capture.  GEMM launches on one device share the scratch: they must
-// not overlap in time.
-hipError_t prepare_gemm_fp32();
+// Scratch of the GEMM's K-split path: partial tiles and their arrival counters (zero between launches).
+// Launches that share a scratch must not overlap in time.
+struct GemmScratch {
+    float* partials = nullptr;
+    unsigned* arrivals = nullptr;
+    int max_partials = 0;
+};
+hipError_t gemm_scratch_create(GemmScratch* out);  // 64 MiB + counters on the current device
+void gemm_scratch_destroy(GemmScratch* ws);
+// The scratch that belongs to stream s on the current device, created at the first call for that stream
+// (which therefore must not come while s is being captured: hipErrorStreamCaptureUnsupported).
+hipError_t gemm_scratch_for_stream(hipStream_t s, GemmScratch* out);
+// Partial tiles the schedule of an M x N x K call parks (0: no K split); -1 if the device cannot be queried.
+int gemm_partial_tiles(int M, int N, int K);
+// hipErrorInvalidValue if the call's schedule needs more partial tiles than ws holds.
+hipError_t launch_gemm_fp32(const void* A, const void* B, float* C, int M, int N, int K, const GemmScratch& ws, hipStream_t s);
+// Walks the work list of a launch on the host (wm = 1: 32 x 128 tiles, 2: 64 x 64) for a device with
+// slots_fit resident workgroups on cus CUs: >= 0 (the partial tiles used) if every tile and chunk is
+// covered exactly once and no partial tile is shared, else a negative code.
+int gemm_schedule_selfcheck(int M, int N, int K, int slots_fit, int cus, int wm);
 // Few-row variant (M <= 8, activation rows resident in LDS, no matrix cores), used by
 // launch_gemm_fp32 when gemm_rows_fits(): same arguments and results within the same tolerance.
 bool gemm_rows_fits(int M, int K);
@@ -68,8 +99,14 @@ hipError_t launch_gemv_a80w40(const void* A, const void* B, float* C, int N, int
 // scaled sum = d_a * sum(q) (both exact), then contracted by launch_gemm_fp32.
 size_t gemm_a80w40_workspace_bytes(int M, int N, int K);
 hipError_t launch_gemm_a80w40(const void* A, const void* B, float* C, int M, int N, int K, void* workspace,
-                              hipStream_t s);
+                              const GemmScratch& ws, hipStream_t s);
 
+
+}  // namespace a81w41
+struct a81w41_context;
+namespace a81w41 {
+// The K-split scratch a context owns (capi.cpp).
+const GemmScratch& context_gemm_scratch(const a81w41_context* ctx);
 
 // Records `message` as the calling thread's last error and returns `status` (capi.cpp).
 int report_failure(int status, const char* message);

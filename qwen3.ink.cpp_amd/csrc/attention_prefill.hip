@@ -383,11 +383,8 @@ hipError_t launch_attention_prefill(const float* q, int q_row_stride, const void
     // leaves most of the chip idle (322 tokens, 8 KV heads: 88 workgroups), so the group is then cut
     // into workgroups of fewer heads and more key splits until there are at least 128 (322 tokens: 23.6 -> 21.2 us
     // with two heads per workgroup; one head per workgroup: 32.6 us, and 10.2 against 11.3 us at 64 tokens).
-    // A81W41_ATTENTION_HEADS=<G> fixes the heads per workgroup (measurement aid).
-    static const int env_g = [] {
-        const char* e = getenv("A81W41_ATTENTION_HEADS");
-        return e ? atoi(e) : 0;
-    }();
+    // A81W41_ATTENTION_HEADS=<G> fixes the heads per workgroup (measurement aid, tuning builds only).
+    static const int env_g = tuning_env_int("A81W41_ATTENTION_HEADS");
     int g = group;
     while (g > 1 && tiles * n_kv * (group / g) < 128) g >>= 1;
     if (env_g > 0 && env_g <= group && group % env_g == 0) g = env_g;

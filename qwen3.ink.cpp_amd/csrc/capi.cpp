@@ -129,6 +129,7 @@ int check_device() {
 }  // namespace
 
 struct a81w41_context {
+    a81w41::GemmScratch gemm_scratch;  // partial tiles of the GEMM's K split: this context's own
     void* act_scratch = nullptr;  // quantised activations, sized for the fp32 layout
     size_t act_bytes = 0;
     int64_t max_elems = 0;
@@ -145,6 +146,7 @@ struct a81w41_linear {
 };
 
 namespace a81w41 {
+const GemmScratch& context_gemm_scratch(const a81w41_context* ctx) { return ctx->gemm_scratch; }
 // Lets the other translation units of the library leave their message where a81w41_last_error() finds it.
 int report_failure(int status, const char* message) { return fail(status, "%s", message); }
 uint16_t float_to_half_bits(float f) { return f32_to_f16(f); }
@@ -280,6 +282,20 @@ int a81w41_quantize_row_q8_1_repack_fp32(const float* x_dev, void* vy_dev, int64
     return quantize_checked(true, x_dev, vy_dev, k, stream);
 }
 
+// The K-split scratch of the free-standing GEMM entry points: one per stream, so that calls on different
+// streams never share partial tiles; none is needed (or created) for calls that do not split K.
+static int stream_scratch(void* stream, int M, int N, int K, a81w41::GemmScratch* ws) {
+    if (a81w41::gemm_partial_tiles(M, N, K) == 0) return A81W41_OK;
+    const hipError_t e = a81w41::gemm_scratch_for_stream(static_cast<hipStream_t>(stream), ws);
+    if (e == hipErrorStreamCaptureUnsupported)
+        return fail(A81W41_ERR_INVALID_ARG,
+                    "the first K-split GEMM call on a stream allocates that stream's scratch and cannot be captured: "
+                    "call once before the capture or use a layer object");
+    if (e == hipErrorOutOfMemory) return fail(A81W41_ERR_HIP, "GEMM scratch: out of device memory or more than 16 streams");
+    if (e != hipSuccess) return hip_fail(e, "gemm_scratch_for_stream");
+    return A81W41_OK;
+}
+
 static int contract_args_ok(const void* A, const void* B, const void* C, int M, int N, int K) {
     if (M < 1) return fail(A81W41_ERR_INVALID_ARG, "M must be >= 1, got %d", M);
     if (!shape_ok(N, K)) return fail(A81W41_ERR_INVALID_ARG, "need K %% 64 == 0 and N %% 8 == 0, got K=%d N=%d", K, N);
@@ -305,8 +321,16 @@ int a81w41_gemm_repack_A81W41_fp32(const void* A_repack_dev, const void* B_repac
     if (int st = contract_args_ok(A_repack_dev, B_repack_dev, C_dev, M, N, K)) return st;
     if (reinterpret_cast<uintptr_t>(A_repack_dev) & 15)
         return fail(A81W41_ERR_INVALID_ARG, "activation blob must be 16-byte aligned");
-    HIP_TRY(a81w41::launch_gemm_fp32(A_repack_dev, B_repack_dev, C_dev, M, N, K, static_cast<hipStream_t>(stream)));
+    a81w41::GemmScratch ws;
+    if (int st = stream_scratch(stream, M, N, K, &ws)) return st;
+    HIP_TRY(a81w41::launch_gemm_fp32(A_repack_dev, B_repack_dev, C_dev, M, N, K, ws, static_cast<hipStream_t>(stream)));
     return A81W41_OK;
+}
+
+int a81w41_gemm_schedule_selfcheck(int M, int N, int K, int resident_workgroups, int cus, int tile) {
+    if (M < 1 || !shape_ok(N, K) || cus < 1 || resident_workgroups < cus || resident_workgroups % cus || (tile != 1 && tile != 2))
+        return fail(A81W41_ERR_INVALID_ARG, "bad arguments") * -100;
+    return a81w41::gemm_schedule_selfcheck(M, N, K, resident_workgroups, cus, tile);
 }
 
 int a81w41_gemv_repack_A80W40(const void* A_repack_dev, const void* B_repack_dev, float* C_dev, int M, int N,
@@ -336,7 +360,9 @@ int a81w41_gemm_repack_A80W40(const void* A_repack_dev, const void* B_repack_dev
     if (workspace_bytes < need)
         return fail(A81W41_ERR_INVALID_ARG, "workspace of %zu bytes is too small, M=%d N=%d K=%d needs %zu", workspace_bytes,
                     M, N, K, need);
-    HIP_TRY(a81w41::launch_gemm_a80w40(A_repack_dev, B_repack_dev, C_dev, M, N, K, workspace_dev,
+    a81w41::GemmScratch ws;
+    if (int st = stream_scratch(stream, M, N, K, &ws)) return st;
+    HIP_TRY(a81w41::launch_gemm_a80w40(A_repack_dev, B_repack_dev, C_dev, M, N, K, workspace_dev, ws,
                                        static_cast<hipStream_t>(stream)));
     return A81W41_OK;
 }
@@ -367,14 +393,18 @@ int a81w41_context_create(int max_rows, int max_cols, a81w41_context** out) {
     if (!ctx) return fail(A81W41_ERR_HIP, "out of host memory");
     ctx->max_elems = (int64_t)max_rows * max_cols;
     ctx->act_bytes = (size_t)(ctx->max_elems / 64) * a81w41::kABlock32;
-    HIP_TRY(a81w41::prepare_gemm_fp32());  // so that a first forward may run inside a stream capture
-    HIP_TRY(hipMalloc(&ctx->act_scratch, ctx->act_bytes));
+    HIP_TRY(a81w41::gemm_scratch_create(&ctx->gemm_scratch));
+    if (hipError_t e = hipMalloc(&ctx->act_scratch, ctx->act_bytes); e != hipSuccess) {
+        a81w41::gemm_scratch_destroy(&ctx->gemm_scratch);
+        return hip_fail(e, "hipMalloc(activation scratch)");
+    }
     *out = ctx.release();
     return A81W41_OK;
 }
 
 void a81w41_context_destroy(a81w41_context* ctx) {
     if (!ctx) return;
+    a81w41::gemm_scratch_destroy(&ctx->gemm_scratch);
     (void)hipFree(ctx->act_scratch);
     (void)hipFree(ctx->x_stage);
     (void)hipFree(ctx->y_stage);
@@ -474,7 +504,10 @@ int a81w41_linear_forward(a81w41_linear* l, const float* x_dev, int M, float* y_
     if (M > 1) {
         if (!l->w32) return fail(A81W41_ERR_INVALID_ARG, "layer has no fp32-parameter blob (needed for M > 1)");
         if (int st = a81w41_quantize_row_q8_1_repack_fp32(x_dev, ctx->act_scratch, (int64_t)M * l->K, stream)) return st;
-        return a81w41_gemm_repack_A81W41_fp32(ctx->act_scratch, l->w32, y_dev, M, l->N, l->K, stream);
+        if (int st = contract_args_ok(ctx->act_scratch, l->w32, y_dev, M, l->N, l->K)) return st;
+        HIP_TRY(a81w41::launch_gemm_fp32(ctx->act_scratch, l->w32, y_dev, M, l->N, l->K, ctx->gemm_scratch,
+                                         static_cast<hipStream_t>(stream)));
+        return A81W41_OK;
     }
     if (!l->w16) return fail(A81W41_ERR_INVALID_ARG, "layer has no fp16-parameter blob (needed for M == 1)");
     if ((reinterpret_cast<uintptr_t>(x_dev) & 15) == 0 && a81w41::gemv_lds_bytes(l->K) <= a81w41::kLdsLimitBytes) {

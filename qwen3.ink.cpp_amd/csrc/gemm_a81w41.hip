@@ -43,6 +43,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <mutex>
+#include <vector>
 
 namespace a81w41 {
 namespace gemm_detail {
@@ -198,7 +199,7 @@ struct Schedule {
 // XCD's column panels wide, row tiles of a panel next to each other.  The workgroups of an XCD that
 // run at the same time then share about band rows' activations and 128 / band panels' weights in its
 // L2, instead of every row tile's activations against two panels when there are many row tiles.
-__device__ __forceinline__ void tile_xy(int tau, int tiles_m, int tiles_n, int band, int& x, int& y) {
+__host__ __device__ __forceinline__ void tile_xy(int tau, int tiles_m, int tiles_n, int band, int& x, int& y) {
     const int tn8 = tiles_n & ~7, main_tiles = tn8 * tiles_m;
     if (tau < main_tiles) {
         const int c = tau & 7, j = tau >> 3;
@@ -438,27 +439,35 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
     tile_kernel_body<1>(A, B, C, M, N, nb_k, sc, partials, arrivals, lds, s_arrived);
 }
 
-// Scratch of the K-split path, one per device, allocated on first use and kept for the life of
-// the process: kMaxPartials partial tiles (64 MiB) and as many arrival counters (zero between launches).
-constexpr int kMaxPartials = 4096;
+// ---- scratch of the K-split path --------------------------------------------------------------
+// A scratch is `max_partials` partial tiles of kPartialWords floats plus as many arrival counters, which
+// are zero between launches.  Launches that share a scratch must not overlap in time, so every owner
+// has its own: a context (all of its layers' calls), a stream (the free-standing GEMM entry point: calls
+// on one stream are ordered by the stream, calls on different streams get different scratches).
+constexpr int kMaxPartials = 4096;  // room for every tile of a launch that does not fill the chip to be cut in four
 constexpr int kMaxDevices = 64;
-struct SplitScratch {
-    float* partials = nullptr;
-    unsigned* arrivals = nullptr;
+constexpr int kMaxStreamsPerDevice = 16;
+
+struct DeviceInfo {
     int slots = 0;  // workgroups of the tile kernels the device holds at once (four per CU)
     int cus = 0;
+    struct {
+        hipStream_t stream;
+        GemmScratch ws;
+    } by_stream[kMaxStreamsPerDevice];
+    int n_streams = 0;
 };
-SplitScratch g_scratch[kMaxDevices];
-std::mutex g_scratch_mutex;
+DeviceInfo g_dev[kMaxDevices];
+std::mutex g_dev_mutex;
 
-hipError_t split_scratch(SplitScratch& out) {
+// Occupancy and CU count of the current device (queried once per device); g_dev_mutex held.
+hipError_t device_info_locked(DeviceInfo*& out) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
-    std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    SplitScratch& s = g_scratch[dev];
-    if (s.slots == 0) {
+    DeviceInfo& d = g_dev[dev];
+    if (d.slots == 0) {
         int per_cu = 0, per_cu_small = 0, cus = 0;
         e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(&gemm_a81w41_tile64_kernel),
                                                          kTileThreads, Geom<2>::kLdsBytes);
@@ -471,34 +480,18 @@ hipError_t split_scratch(SplitScratch& out) {
         e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
         if (e != hipSuccess) return e;
         if (per_cu < 1 || cus < 1) return hipErrorInvalidValue;
-        float* p = nullptr;
-        unsigned* a = nullptr;
-        e = hipMalloc(&p, (size_t)kMaxPartials * kPartialWords * sizeof(float));
-        if (e != hipSuccess) return e;
-        e = hipMalloc(&a, kMaxPartials * sizeof(unsigned));
-        if (e == hipSuccess) e = hipMemset(a, 0, kMaxPartials * sizeof(unsigned));
-        if (e != hipSuccess) {
-            (void)hipFree(p);
-            (void)hipFree(a);
-            return e;
-        }
-        s.partials = p;
-        s.arrivals = a;
-        s.slots = per_cu * cus;
-        s.cus = cus;
+        d.cus = cus;
+        d.slots = per_cu * cus;
     }
-    out = s;
+    out = &d;
     return hipSuccess;
 }
 
-// WM = 2: 64 x 64 tiles; WM = 1: 32 x 128 tiles (calls with at most 32 rows).
+// The schedule of one launch (see Schedule): a pure function of the shape and of the device's size.
+// Returns false when the K split the shape calls for needs more than max_partials partial tiles.
 template <int WM>
-hipError_t launch_tiles(const void* A, const void* B, float* C, int M, int N, int K, hipStream_t s) {
-    SplitScratch ws;
-    hipError_t e = split_scratch(ws);
-    if (e != hipSuccess) return e;
+bool make_schedule(int M, int N, int K, int slots_fit, int cus, int max_partials, Schedule& sc, int& grid) {
     const int nb_k = K / 64;
-    Schedule sc;
     sc.tiles_m = (M + Geom<WM>::kTileM - 1) / Geom<WM>::kTileM;
     sc.tiles_n = (N + Geom<WM>::kTileN - 1) / Geom<WM>::kTileN;
     const int T = sc.tiles_m * sc.tiles_n;
@@ -506,33 +499,23 @@ hipError_t launch_tiles(const void* A, const void* B, float* C, int M, int N, in
     // tiles T per CU (measured at N = 4096, M = 128..1536): up to 2 per CU, four (finer K split over
     // more workgroups); up to 2.67, two (one round of two-per-CU tiles plus a split remainder beats a
     // sparse round of slower ones: 640 rows 144 against 155 us); up to 4, three (832 rows 179 against
-    // 201 us); from 4 on, four.  A81W41_GEMM_PER_CU=<n> fixes the figure (measurement aid).
-    static const int env_per_cu = [] {
-        const char* v = getenv("A81W41_GEMM_PER_CU");
-        return v ? atoi(v) : 0;
-    }();
-    const int fit = ws.slots / ws.cus;
+    // 201 us); from 4 on, four.
+    const int fit = slots_fit / cus;
     int per_cu = fit;
-    if (T > 2 * ws.cus && T < 4 * ws.cus) per_cu = 3 * T <= 8 * ws.cus ? 2 : 3;
+    if (T > 2 * cus && T < 4 * cus) per_cu = 3 * T <= 8 * cus ? 2 : 3;
     if (per_cu > fit) per_cu = fit;
+    const int env_per_cu = tuning_env_int("A81W41_GEMM_PER_CU");
     if (env_per_cu >= 1 && env_per_cu <= fit) per_cu = env_per_cu;
-    ws.slots = per_cu * ws.cus;
-    sc.whole = (T / ws.slots) * ws.slots;
+    const int slots = per_cu * cus;
+    sc.whole = (T / slots) * slots;
     sc.r = T - sc.whole;
     // Split the last, partial round: in two, so that the chunks go to the first (faster) half
     // of the grid; in four when even then less than 3/4 of the grid would have one.
-    // A81W41_GEMM_SPLIT=<c> overrides (measurement aid; ignored unless valid).
-    static const int env_c = [] {
-        const char* v = getenv("A81W41_GEMM_SPLIT");
-        return v ? atoi(v) : 0;
-    }();
     int c = 1;
-    auto valid = [&](int cc) {
-        return cc >= 1 && cc <= 16 && nb_k % (Geom<WM>::kRing * cc) == 0 && (long long)sc.r * cc <= kMaxPartials;
-    };
+    auto valid = [&](int cc) { return cc >= 1 && cc <= 16 && nb_k % (Geom<WM>::kRing * cc) == 0 && (long long)sc.r * cc <= kMaxPartials; };
     if (sc.r > 0) {
         if (valid(2)) c = 2;
-        if (valid(4) && sc.r * 4 <= ws.slots * 3 / 4) c = 4;
+        if (valid(4) && sc.r * 4 <= slots * 3 / 4) c = 4;
         // a launch that does not fill the chip once, over a long K: quarters still leave 48 steps per chunk
         // (down_proj at 322 rows: 75.6 against 79.8 us)
         if (valid(4) && sc.whole == 0 && nb_k / 4 >= 48) c = 4;
@@ -541,26 +524,40 @@ hipError_t launch_tiles(const void* A, const void* B, float* C, int M, int N, in
             // weights once, so cut K as finely as still leaves 8 super-blocks per chunk and one chunk
             // per workgroup slot.
             for (int cc : {6, 8, 12, 16})
-                if (valid(cc) && nb_k / cc >= 8 && sc.r * cc <= ws.slots) c = cc;
+                if (valid(cc) && nb_k / cc >= 8 && sc.r * cc <= slots) c = cc;
         }
+        const int env_c = tuning_env_int("A81W41_GEMM_SPLIT");
         if (env_c > 0 && valid(env_c)) c = env_c;
     }
     if (c == 1) {
         sc.whole = T;
         sc.r = 0;
     }
-    static const int env_band = [] {
-        const char* v = getenv("A81W41_GEMM_BAND");
-        return v ? atoi(v) : 0;
-    }();
     // Bands of 4 row tiles: neutral up to 16 row tiles, 5-8 % faster from 24 on (gate at 4096 rows: 860 -> 807 us;
-    // 2, 3, 6 and 8 measured the same within noise).  A81W41_GEMM_BAND=<rows> overrides (measurement aid).
+    // 2, 3, 6 and 8 measured the same within noise).
     sc.band = sc.tiles_m < 4 ? sc.tiles_m : 4;
+    const int env_band = tuning_env_int("A81W41_GEMM_BAND");
     if (env_band > 0) sc.band = env_band < sc.tiles_m ? env_band : sc.tiles_m;
     sc.c = c;
     sc.chunk = nb_k / c;
     sc.items = sc.whole + sc.r * c;
-    const int grid = sc.items < ws.slots ? sc.items : ws.slots;
+    grid = sc.items < slots ? sc.items : slots;
+    return sc.r * c <= max_partials;
+}
+
+// WM = 2: 64 x 64 tiles; WM = 1: 32 x 128 tiles (calls with at most 32 rows).
+template <int WM>
+hipError_t launch_tiles(const void* A, const void* B, float* C, int M, int N, int K, const GemmScratch& ws, hipStream_t s) {
+    DeviceInfo* d = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_dev_mutex);
+        const hipError_t e = device_info_locked(d);
+        if (e != hipSuccess) return e;
+    }
+    Schedule sc;
+    int grid = 0;
+    if (!make_schedule<WM>(M, N, K, d->slots, d->cus, ws.max_partials, sc, grid)) return hipErrorInvalidValue;
+    const int nb_k = K / 64;
     if (WM == 2)
         hipLaunchKernelGGL(gemm_a81w41_tile64_kernel, dim3(grid), dim3(kTileThreads), Geom<2>::kLdsBytes, s,
                            static_cast<const uint8_t*>(A), static_cast<const uint8_t*>(B), M, N, nb_k, sc.tiles_m,
@@ -573,33 +570,137 @@ hipError_t launch_tiles(const void* A, const void* B, float* C, int M, int N, in
     return hipGetLastError();
 }
 
+// Which kernel a call goes to: 0 the few-row kernel (no scratch), 1 the 32 x 128 tiles, 2 the 64 x 64 tiles.
+int pick_kernel(int M, int N, int K) {
+    // Measurement aids (tuning builds): A81W41_GEMM_TUNE=tile keeps few-row calls on the matrix-core kernels,
+    // A81W41_GEMM_TUNE=Tile64 additionally keeps every call on the 64 x 64 arrangement.
+    const char* tune_s = tuning_env("A81W41_GEMM_TUNE");
+    const char tune = tune_s ? tune_s[0] : '\0';
+    const bool tile_only = tune == 't' || tune == 'T';
+    if (!tile_only && gemm_rows_fits(M, K)) return 0;
+    // At most 32 rows: 32 x 128 tiles (no wave idles on rows that do not exist).  Measured at M = 9..32 with
+    // the four-per-CU kernels: N = 12288 17 us against 22 us with 64 x 64 tiles, down_proj (N = 4096,
+    // K = 12288) 21.2 against 24.5, N = 4096 and 1024 at K = 4096 equal.
+    const int env_n = tuning_env_int("A81W41_GEMM_N32X128");
+    const int min_n_32x128 = env_n > 0 ? env_n : 1024;
+    if (M <= 32 && N >= min_n_32x128 && tune != 'T') return 1;
+    return 2;
+}
+
 }  // namespace gemm_detail
 
 using namespace gemm_detail;
 
-hipError_t prepare_gemm_fp32() {
-    SplitScratch ws;
-    return split_scratch(ws);
+hipError_t gemm_scratch_create(GemmScratch* out) {
+    out->partials = nullptr;
+    out->arrivals = nullptr;
+    out->max_partials = 0;
+    float* p = nullptr;
+    unsigned* a = nullptr;
+    hipError_t e = hipMalloc(&p, (size_t)kMaxPartials * kPartialWords * sizeof(float));
+    if (e != hipSuccess) return e;
+    e = hipMalloc(&a, kMaxPartials * sizeof(unsigned));
+    if (e == hipSuccess) e = hipMemset(a, 0, kMaxPartials * sizeof(unsigned));
+    if (e != hipSuccess) {
+        (void)hipFree(p);
+        (void)hipFree(a);
+        return e;
+    }
+    out->partials = p;
+    out->arrivals = a;
+    out->max_partials = kMaxPartials;
+    return hipSuccess;
 }
 
-hipError_t launch_gemm_fp32(const void* A, const void* B, float* C, int M, int N, int K, hipStream_t s) {
-    // Measurement aids: A81W41_GEMM_TUNE=tile keeps few-row calls on the matrix-core kernels,
-    // A81W41_GEMM_TUNE=Tile64 additionally keeps every call on the 64 x 64 arrangement.
-    static const char tune = [] {
-        const char* e = getenv("A81W41_GEMM_TUNE");
-        return e ? e[0] : '\0';
-    }();
-    const bool tile_only = tune == 't' || tune == 'T';
-    if (!tile_only && gemm_rows_fits(M, K)) return launch_gemm_rows_fp32(A, B, C, M, N, K, s);
-    // At most 32 rows: 32 x 128 tiles (no wave idles on rows that do not exist).  Measured at M = 9..32 with
-    // the four-per-CU kernels: N = 12288 17 us against 22 us with 64 x 64 tiles, down_proj (N = 4096,
-    // K = 12288) 21.2 against 24.5, N = 4096 and 1024 at K = 4096 equal.
-    static const int min_n_32x128 = [] {
-        const char* e = getenv("A81W41_GEMM_N32X128");
-        return e ? atoi(e) : 1024;
-    }();
-    if (M <= 32 && N >= min_n_32x128 && tune != 'T') return launch_tiles<1>(A, B, C, M, N, K, s);
-    return launch_tiles<2>(A, B, C, M, N, K, s);
+void gemm_scratch_destroy(GemmScratch* ws) {
+    (void)hipFree(ws->partials);
+    (void)hipFree(ws->arrivals);
+    ws->partials = nullptr;
+    ws->arrivals = nullptr;
+    ws->max_partials = 0;
+}
+
+hipError_t gemm_scratch_for_stream(hipStream_t s, GemmScratch* out) {
+    std::lock_guard<std::mutex> lock(g_dev_mutex);
+    DeviceInfo* d = nullptr;
+    hipError_t e = device_info_locked(d);
+    if (e != hipSuccess) return e;
+    for (int i = 0; i < d->n_streams; i++)
+        if (d->by_stream[i].stream == s) {
+            *out = d->by_stream[i].ws;
+            return hipSuccess;
+        }
+    if (d->n_streams == kMaxStreamsPerDevice) return hipErrorOutOfMemory;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    e = hipStreamIsCapturing(s, &cap);
+    if (e != hipSuccess) return e;
+    if (cap != hipStreamCaptureStatusNone) return hipErrorStreamCaptureUnsupported;  // cannot allocate under capture
+    GemmScratch ws;
+    e = gemm_scratch_create(&ws);
+    if (e != hipSuccess) return e;
+    d->by_stream[d->n_streams].stream = s;
+    d->by_stream[d->n_streams].ws = ws;
+    d->n_streams++;
+    *out = ws;
+    return hipSuccess;
+}
+
+int gemm_partial_tiles(int M, int N, int K) {
+    const int kernel = pick_kernel(M, N, K);
+    if (kernel == 0) return 0;
+    std::lock_guard<std::mutex> lock(g_dev_mutex);
+    DeviceInfo* d = nullptr;
+    if (device_info_locked(d) != hipSuccess) return -1;
+    Schedule sc;
+    int grid = 0;
+    if (kernel == 1)
+        make_schedule<1>(M, N, K, d->slots, d->cus, kMaxPartials, sc, grid);
+    else
+        make_schedule<2>(M, N, K, d->slots, d->cus, kMaxPartials, sc, grid);
+    return sc.r * sc.c;
+}
+
+hipError_t launch_gemm_fp32(const void* A, const void* B, float* C, int M, int N, int K, const GemmScratch& ws, hipStream_t s) {
+    switch (pick_kernel(M, N, K)) {
+        case 0: return launch_gemm_rows_fp32(A, B, C, M, N, K, s);
+        case 1: return launch_tiles<1>(A, B, C, M, N, K, ws, s);
+        default: return launch_tiles<2>(A, B, C, M, N, K, ws, s);
+    }
+}
+
+// Host-side check of the work list a launch would walk (no device needed): every whole tile once, every
+// chunk of every split tile once, partial-tile indices distinct and below the scratch size.
+int gemm_schedule_selfcheck(int M, int N, int K, int slots_fit, int cus, int wm) {
+    Schedule sc;
+    int grid = 0;
+    const bool fits = wm == 1 ? make_schedule<1>(M, N, K, slots_fit, cus, kMaxPartials, sc, grid)
+                              : make_schedule<2>(M, N, K, slots_fit, cus, kMaxPartials, sc, grid);
+    if (!fits) return -1;
+    const int T = sc.tiles_m * sc.tiles_n, nb_k = K / 64;
+    if (sc.whole + sc.r != T || sc.items != sc.whole + sc.r * sc.c || sc.chunk * sc.c != nb_k) return -2;
+    if (grid < 1 || grid > slots_fit) return -3;
+    std::vector<int> covered((size_t)T, 0), part_used((size_t)kMaxPartials, 0);
+    for (int b = 0; b < grid; b++)
+        for (int item = b; item < sc.items; item += grid) {
+            if (item < sc.whole) {
+                covered[item] += nb_k;
+            } else {
+                const int k = item - sc.whole, tr = k % sc.r, ch = k / sc.r, part = tr * sc.c + ch;
+                if (part < 0 || part >= kMaxPartials || part_used[part]++) return -4;
+                if (ch * sc.chunk + sc.chunk > nb_k) return -5;
+                covered[sc.whole + tr] += sc.chunk;
+            }
+        }
+    for (int t = 0; t < T; t++)
+        if (covered[t] != nb_k) return -6;
+    // the tile numbering is one-to-one onto the tiles
+    std::vector<int> seen((size_t)T, 0);
+    for (int tau = 0; tau < T; tau++) {
+        int x = -1, y = -1;
+        tile_xy(tau, sc.tiles_m, sc.tiles_n, sc.band, x, y);
+        if (x < 0 || x >= sc.tiles_n || y < 0 || y >= sc.tiles_m || seen[(size_t)y * sc.tiles_n + x]++) return -7;
+    }
+    return sc.r * sc.c;
 }
 
 }  // namespace a81w41

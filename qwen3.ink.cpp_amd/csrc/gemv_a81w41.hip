@@ -445,12 +445,12 @@ struct GemvTune {
     int waves, max_grid, wpg;  // workgroup width, persistent-grid cap, waves per column group (0 = auto)
 };
 
-// Workgroup width and persistent-grid cap.  A81W41_GEMV_TUNE="waves,grid" overrides
+// Workgroup width and persistent-grid cap.  In tuning builds A81W41_GEMV_TUNE="waves,grid,wpg" overrides
 // the table (measurement aid; waves must be 4, 8 or 16).
 GemvTune pick_tune(int nb_n, int nb_k) {
     static const GemvTune env = [] {
         GemvTune t{0, 0, 0};
-        if (const char* e = getenv("A81W41_GEMV_TUNE")) sscanf(e, "%d,%d,%d", &t.waves, &t.max_grid, &t.wpg);
+        if (const char* e = tuning_env("A81W41_GEMV_TUNE")) sscanf(e, "%d,%d,%d", &t.waves, &t.max_grid, &t.wpg);
         return t;
     }();
     if (env.waves == 4 || env.waves == 8 || env.waves == 16)
@@ -492,11 +492,15 @@ hipError_t launch(const void* a_or_x, void* a_out, int n_mat, const void* const*
     int wpg_log2 = 0;
     const int want = t.wpg > 0 ? t.wpg : n_steps;
     while ((2 << wpg_log2) <= want && (2 << wpg_log2) <= t.waves) wpg_log2++;
+    // paired output: a workgroup walks its eight groups in 8 / slots rounds, so at most eight groups at a time
+    // (short rows in wide workgroups -- hidden 1024 with 16 waves -- would otherwise have sixteen)
+    if (PRO == kProAddNormPair)
+        while ((t.waves >> wpg_log2) > 8) wpg_log2++;
     const int slots = t.waves >> wpg_log2;
     const int wgs = (nb_n + slots - 1) / slots;
     int grid = wgs < t.max_grid ? wgs : t.max_grid;
     if (PRO == kProAddNormPair) {  // one workgroup per 32-block of the paired output
-        if (n_mat != 1 || nb_n % 8 || slots > 8 || pro.pair_out == nullptr) return hipErrorInvalidValue;
+        if (n_mat != 1 || nb_n % 8 || pro.pair_out == nullptr) return hipErrorInvalidValue;
         grid = nb_n / 8;
     }
     uint8_t* ao = static_cast<uint8_t*>(a_out);
@@ -546,6 +550,8 @@ hipError_t launch_gemv_add_norm(const float* x, const GemvPrologue& pro, void* a
                                 int K, hipStream_t s) {
     return launch<kProAddNorm>(x, a_out, 1, &B, &C, &N, K, pro, s);
 }
+
+bool gemv_pair_fits(int N, int K) { return gemv_add_norm_fits(K) && N % 64 == 0; }
 
 hipError_t launch_gemv_add_norm_silu_pair(const float* x, const GemvPrologue& pro, const void* B_gate_up, int N, int K,
                                           hipStream_t s) {

@@ -37,7 +37,6 @@ int fail(int status, const char* fmt, ...) {
     } while (0)
 
 constexpr int kHeadDim = 128;
-constexpr int kCuCount = 256;  // MI355X
 
 struct LayerWeights {
     a81w41_linear* lin[4] = {nullptr, nullptr, nullptr, nullptr};  // qkv, o, gate_up, down
@@ -67,6 +66,11 @@ struct a81w41_qwen3 {
     unsigned* attn_arrive = nullptr;  // ... and n_q arrival counters, zero between launches
     float attn_scale = 0.f;  // 1/sqrt(128) unless a scaling.bin said otherwise
     hipStream_t stream = nullptr;
+    int cu_count = 0;  // of the device the model lives on
+    // Switches of a81w41_qwen3_set_option: each keeps a fusion off (or fixes the attention's key split) so
+    // that tests can compare the fused pass with the separate kernels bit for bit.
+    bool opt_unfused = false, opt_attn_fp32 = false, opt_no_pair = false, opt_vector_attention = false;
+    int opt_attention_split = 0;
     int qkv_dim() const { return (cfg.n_q_heads + 2 * cfg.n_kv_heads) * kHeadDim; }
 };
 
@@ -121,15 +125,15 @@ int enqueue_pass(a81w41_qwen3* m, int M, hipStream_t s) {
     // linear's own quantiser would produce from the fp32 rows, which therefore never go to memory.
     const bool quant_fused = M > 1 && prefill_fusion_usable(m);
     void* scratch = a81w41_context_activation_scratch_dev(m->ctx);
-    static const bool vector_attention = getenv("A81W41_ATTENTION_VECTOR") != nullptr;  // measurement aid, see launch_attention
-    const bool attn_blocks = !vector_attention && a81w41::attention_prefill_fits(M, c.n_q_heads, c.n_kv_heads);
+    const a81w41::GemmScratch& gws = a81w41::context_gemm_scratch(m->ctx);
+    const bool attn_blocks = !m->opt_vector_attention && a81w41::attention_prefill_fits(M, c.n_q_heads, c.n_kv_heads);
     for (int l = 0; l < c.n_layers; l++) {
         LayerWeights& L = m->layers[l];
         const float* norm_in = pending ? pending : m->x;
         const float* norm_res = pending ? m->x : nullptr;
         if (quant_fused) {
             Q_HIP(a81w41::launch_add_rmsnorm_quant(norm_in, norm_res, L.norm[0], m->x, scratch, M, c.hidden, c.rms_eps, s));
-            Q_HIP(a81w41::launch_gemm_fp32(scratch, a81w41_linear_weight_fp32_dev(L.lin[0]), m->qkv, M, qkv_dim, c.hidden, s));
+            Q_HIP(a81w41::launch_gemm_fp32(scratch, a81w41_linear_weight_fp32_dev(L.lin[0]), m->qkv, M, qkv_dim, c.hidden, gws, s));
         } else {
             Q_HIP(a81w41::launch_add_rmsnorm(norm_in, norm_res, L.norm[0], m->x, m->h, M, c.hidden, c.rms_eps, s));
             Q_TRY(a81w41_linear_forward(L.lin[0], m->h, M, m->qkv, s));
@@ -139,18 +143,18 @@ int enqueue_pass(a81w41_qwen3* m, int M, hipStream_t s) {
         if (quant_fused && attn_blocks) {  // the matrix-core attention hands o_proj its input as quantised blocks
             Q_HIP(a81w41::launch_attention_prefill(m->qkv, qkv_dim, L.k_cache, L.v_cache, m->pos, nullptr, q_dim, M, c.n_q_heads,
                                                    c.n_kv_heads, c.max_seq, scale, s, scratch));
-            Q_HIP(a81w41::launch_gemm_fp32(scratch, a81w41_linear_weight_fp32_dev(L.lin[1]), m->o, M, c.hidden, q_dim, s));
+            Q_HIP(a81w41::launch_gemm_fp32(scratch, a81w41_linear_weight_fp32_dev(L.lin[1]), m->o, M, c.hidden, q_dim, gws, s));
         } else {
             Q_HIP(a81w41::launch_attention(m->qkv, qkv_dim, L.k_cache, L.v_cache, m->pos, m->attn, q_dim, M, c.n_q_heads,
-                                           c.n_kv_heads, c.max_seq, scale, s));
+                                           c.n_kv_heads, c.max_seq, scale, s, m->opt_vector_attention ? 1 : 0));
             Q_TRY(a81w41_linear_forward(L.lin[1], m->attn, M, m->o, s));
         }
         if (quant_fused) {
             Q_HIP(a81w41::launch_add_rmsnorm_quant(m->o, m->x, L.norm[1], m->x, scratch, M, c.hidden, c.rms_eps, s));
             Q_HIP(a81w41::launch_gemm_fp32(scratch, a81w41_linear_weight_fp32_dev(L.lin[2]), m->gate_up, M, 2 * c.intermediate,
-                                           c.hidden, s));
+                                           c.hidden, gws, s));
             Q_HIP(a81w41::launch_silu_mul_quant(m->gate_up, scratch, M, c.intermediate, s));
-            Q_HIP(a81w41::launch_gemm_fp32(scratch, a81w41_linear_weight_fp32_dev(L.lin[3]), m->o, M, c.hidden, c.intermediate, s));
+            Q_HIP(a81w41::launch_gemm_fp32(scratch, a81w41_linear_weight_fp32_dev(L.lin[3]), m->o, M, c.hidden, c.intermediate, gws, s));
         } else {
             Q_HIP(a81w41::launch_add_rmsnorm(m->o, m->x, L.norm[1], m->x, m->h, M, c.hidden, c.rms_eps, s));
             Q_TRY(a81w41_linear_forward(L.lin[2], m->h, M, m->gate_up, s));
@@ -192,22 +196,17 @@ int enqueue_pass_one_token(a81w41_qwen3* m, hipStream_t s) {
     const int qkv_dim = m->qkv_dim();
     const float scale = m->attn_scale;
     void* scratch = a81w41_context_activation_scratch_dev(m->ctx);
-    // measurement / test aid: attention output as fp32 through o_proj's own quantiser (same bits)
-    static const bool attn_fp32 = getenv("A81W41_QWEN3_ATTN_FP32") != nullptr;
-    // same kind of aid: gate_up writes fp32 and down_proj's prologue does SiLU * mul and the quantising (same bits)
-    static const bool no_pair = getenv("A81W41_QWEN3_NO_PAIR") != nullptr;
+    // test switches (a81w41_qwen3_set_option): attention output as fp32 through o_proj's own quantiser (same
+    // bits); gate_up writes fp32 and down_proj's prologue does SiLU * mul and the quantising (same bits)
+    const bool attn_fp32 = m->opt_attn_fp32, no_pair = m->opt_no_pair || !a81w41::gemv_pair_fits(2 * c.intermediate, c.hidden);
     // Key split of the attention: one workgroup per head, or several shares per head for long contexts.
-    // A81W41_ATTENTION_SPLIT=<1..16> overrides (test and measurement aid).
-    static const int env_split = [] {
-        const char* e = getenv("A81W41_ATTENTION_SPLIT");
-        return e ? atoi(e) : 0;
-    }();
+    const int env_split = m->opt_attention_split;
     // measured (32 query heads, 64 decode steps after the prompt): one share up to about 560 keys, three up
     // to 1280, four up to 2560, then one per 512 keys
     const int ctx = m->plan_ctx;
     int splits = ctx <= 560 ? 1 : ctx <= 1280 ? 3 : ctx <= 2560 ? 4 : (ctx + 511) / 512;
     // ... but no more workgroups than the chip has CUs (a second round of them would cost more than longer shares)
-    const int fit = kCuCount / c.n_q_heads;
+    const int fit = m->cu_count / c.n_q_heads;
     if (splits > fit) splits = fit;
     if (env_split > 0) splits = env_split;
     splits = splits < 1 ? 1 : (splits > a81w41::kAttentionMaxSplits ? a81w41::kAttentionMaxSplits : splits);
@@ -260,8 +259,7 @@ int enqueue_pass_one_token(a81w41_qwen3* m, hipStream_t s) {
 }
 
 bool prefill_fusion_usable(const a81w41_qwen3* m) {
-    static const bool off = getenv("A81W41_QWEN3_UNFUSED") != nullptr;  // measurement aid: keep the separate kernels
-    if (off) return false;
+    if (m->opt_unfused) return false;
     for (const LayerWeights& L : m->layers)
         for (int w = 0; w < 4; w++)
             if (!a81w41_linear_weight_fp32_dev(L.lin[w])) return false;
@@ -269,8 +267,7 @@ bool prefill_fusion_usable(const a81w41_qwen3* m) {
 }
 
 bool one_token_pass_usable(const a81w41_qwen3* m) {
-    static const bool off = getenv("A81W41_QWEN3_UNFUSED") != nullptr;  // measurement aid: keep the separate kernels
-    if (off || !a81w41::gemv_add_norm_fits(m->cfg.hidden)) return false;
+    if (m->opt_unfused || !a81w41::gemv_add_norm_fits(m->cfg.hidden)) return false;
     if (a81w41::gemv_lds_bytes(m->cfg.intermediate) > a81w41::kLdsLimitBytes) return false;
     for (const LayerWeights& L : m->layers)
         for (int w = 0; w < 4; w++)
@@ -302,6 +299,12 @@ int a81w41_qwen3_create(const a81w41_qwen3_config* cfg, a81w41_qwen3** out) {
     if (!m) return fail(A81W41_ERR_HIP, "out of host memory");
     m->cfg = c;
     m->attn_scale = 1.0f / std::sqrt((float)kHeadDim);
+    {
+        int dev = 0;
+        Q_HIP(hipGetDevice(&dev));
+        Q_HIP(hipDeviceGetAttribute(&m->cu_count, hipDeviceAttributeMultiprocessorCount, dev));
+        if (m->cu_count < 1) return fail(A81W41_ERR_HIP, "device reports no compute units");
+    }
     const int max_cols = c.hidden > c.intermediate ? c.hidden : c.intermediate;
     const int q_dim = c.n_q_heads * kHeadDim;
     Q_TRY(a81w41_context_create(c.max_seq, max_cols > q_dim ? max_cols : q_dim, &m->ctx));
@@ -423,6 +426,23 @@ int a81w41_qwen3_set_embedding(a81w41_qwen3* m, const uint16_t* table_fp16) {
     return A81W41_OK;
 }
 
+int a81w41_qwen3_set_option(a81w41_qwen3* m, int option, int value) {
+    if (!m) return fail(A81W41_ERR_INVALID_ARG, "null model");
+    switch (option) {
+        case A81W41_QWEN3_OPT_UNFUSED: m->opt_unfused = value != 0; break;
+        case A81W41_QWEN3_OPT_ATTN_FP32: m->opt_attn_fp32 = value != 0; break;
+        case A81W41_QWEN3_OPT_NO_PAIR: m->opt_no_pair = value != 0; break;
+        case A81W41_QWEN3_OPT_VECTOR_ATTENTION: m->opt_vector_attention = value != 0; break;
+        case A81W41_QWEN3_OPT_ATTENTION_SPLIT:
+            if (value < 0 || value > a81w41::kAttentionMaxSplits)
+                return fail(A81W41_ERR_INVALID_ARG, "attention split must be 0 (automatic) .. %d", a81w41::kAttentionMaxSplits);
+            m->opt_attention_split = value;
+            break;
+        default: return fail(A81W41_ERR_INVALID_ARG, "unknown option %d", option);
+    }
+    return A81W41_OK;
+}
+
 int a81w41_qwen3_reset(a81w41_qwen3* m) {
     if (!m) return fail(A81W41_ERR_INVALID_ARG, "null model");
     Q_HIP(hipStreamSynchronize(m->stream));
@@ -540,7 +560,6 @@ int a81w41_qwen3_generate_greedy(a81w41_qwen3* m, const int* prompt, int n_promp
                 captured = true;
         }
         (void)hipGetLastError();
-        if (getenv("A81W41_DEBUG")) fprintf(stderr, "a81w41: decode step %s\n", captured ? "replayed from a captured graph" : "launched eagerly (capture failed)");
         Q_HIP(hipEventRecord(e3, s));
         for (int i = 0; i < n_steps; i++) {
             if (captured) {

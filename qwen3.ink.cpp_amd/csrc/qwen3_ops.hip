@@ -826,7 +826,7 @@ size_t attention_lds_bytes(int max_seq, int threads) {
 hipError_t launch_attention(const float* q, int q_row_stride, const void* k_cache, const void* v_cache, const int* pos_dev,
                             float* out, int out_row_stride, int M, int n_q, int n_kv, int max_seq, float scale, hipStream_t s,
                             int variant) {
-    static const bool vector_only = getenv("A81W41_ATTENTION_VECTOR") != nullptr;  // measurement aid
+    static const bool vector_only = tuning_env("A81W41_ATTENTION_VECTOR") != nullptr;  // measurement aid (tuning builds)
     if (variant == 0 && !vector_only && attention_prefill_fits(M, n_q, n_kv))
         return launch_attention_prefill(q, q_row_stride, k_cache, v_cache, pos_dev, out, out_row_stride, M, n_q, n_kv, max_seq,
                                         scale, s);

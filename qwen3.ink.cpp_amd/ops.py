@@ -93,8 +93,8 @@ def gemm_fp32(a_blob, b_blob, M: int, N: int, K: int, out=None):
     torch = _torch()
     if out is None:
         out = torch.empty((M, N), dtype=torch.float32, device=a_blob.device)
-    capi.check(capi.lib().a81w41_gemm_repack_A81W41_fp32(_dev_ptr(a_blob), _dev_ptr(b_blob), _dev_ptr(out),
-                                                         M, N, K, _stream()))
+    fn = capi.lib().a81w41_gemm_repack_A81W41_fp32
+    capi.check(fn(_dev_ptr(a_blob), _dev_ptr(b_blob), _dev_ptr(out), M, N, K, _stream()))
     return out
 
 
@@ -357,6 +357,12 @@ class Qwen3Model:
         t = np.ascontiguousarray(table_fp16, np.float16)
         assert t.shape == (self.cfg.vocab, self.cfg.hidden)
         capi.check(capi.lib().a81w41_qwen3_set_embedding(self.handle, t.ctypes.data))
+
+    OPTIONS = {"unfused": 0, "attn_fp32": 1, "no_pair": 2, "vector_attention": 3, "attention_split": 4}
+
+    def set_option(self, name: str, value: int):
+        """Test switch of ``a81w41_qwen3_set_option`` (see include/a81w41.h)."""
+        capi.check(capi.lib().a81w41_qwen3_set_option(self.handle, self.OPTIONS[name], int(value)))
 
     def reset(self):
         capi.check(capi.lib().a81w41_qwen3_reset(self.handle))

@@ -57,7 +57,14 @@ def test_quantize_bit_exact(pkg, ora, synth, torch, fp32, M, K):
 
 
 def test_quantize_special_values(pkg, ora, torch):
-    x = np.zeros((6, 64), np.float32)
+    x = np.zeros((8, 64), np.float32)
+    # 127/amax overflows: q = -128 everywhere, wrapped sum (pinned against x86 in tests/test_oracle_avx2.py)
+    x[6, :32] = np.float32(1e-38) * np.linspace(-1.0, 1.0, 32, dtype=np.float32)
+    x[6, 5] = 0.0
+    x[6, 32:] = np.float32(3e-39)
+    x[6, 40] = 0.0
+    x[7, 17] = np.float32(-2e-38)
+    x[7, 32:] = np.float32(3.8e-37)
     x[1, 7] = 3.5
     x[2, 40] = -2.0
     x[3, :] = 1.0
@@ -350,3 +357,49 @@ def test_forward_m_gt_1_replays_from_a_hip_graph(pkg, ora, synth, torch):
         assert torch.equal(y, eager)
         layer.forward(other)             # eager work between replays, same scratch
         torch.cuda.synchronize()
+
+
+def test_gemm_calls_on_two_streams_do_not_share_partial_tiles(pkg, ora, synth, torch):
+    """K-split GEMM launches that overlap in time on two streams (the free-standing entry point keeps one
+    scratch per stream) and layer calls on two contexts (each owns its scratch): every result equals the
+    one computed alone."""
+    M, N, K = 322, 1024, 4096           # 96 tiles, K cut in four: partial tiles in use
+    cases = []
+    for seed in (501, 503):
+        w4, s, o = synth.weight_files(N, K, seed)
+        x = synth.activations(M, K, seed + 1, outliers=True)
+        ba, bw = ora.quantize(x, True), ora.repack(w4, s, o, K, N, True)
+        a, b = dev(torch, ba), dev(torch, bw)
+        cases.append((a, b, pkg.ops.gemm_fp32(a, b, M, N, K).clone(), dev(torch, x), (w4, s, o)))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [[torch.empty((M, N), dtype=torch.float32, device="cuda") for _ in range(6)] for _ in range(2)]
+    for i, st in enumerate(streams):        # first call on each stream creates its scratch
+        with torch.cuda.stream(st):
+            pkg.ops.gemm_fp32(cases[i][0], cases[i][1], M, N, K, out=outs[i][0])
+    torch.cuda.synchronize()
+    for r in range(6):
+        for i, st in enumerate(streams):
+            with torch.cuda.stream(st):
+                pkg.ops.gemm_fp32(cases[i][0], cases[i][1], M, N, K, out=outs[i][r])
+    torch.cuda.synchronize()
+    for i in range(2):
+        for r in range(6):
+            assert torch.equal(outs[i][r], cases[i][2]), (i, r)
+    # the same through two layer objects on two contexts
+    layers = []
+    for i in range(2):
+        ctx = pkg.ops.Context(max_rows=M, max_cols=K)
+        w4, s, o = cases[i][4]
+        layers.append(pkg.Linear.from_arrays(w4, s, o, N=N, K=K, ctx=ctx))
+    alone = [layers[i].forward(cases[i][3]).clone() for i in range(2)]
+    torch.cuda.synchronize()
+    for r in range(6):
+        for i, st in enumerate(streams):
+            with torch.cuda.stream(st):
+                layers[i].forward(cases[i][3], out=outs[i][r])
+    torch.cuda.synchronize()
+    for i in range(2):
+        assert torch.equal(alone[i], cases[i][2])
+        for r in range(6):
+            assert torch.equal(outs[i][r], alone[i]), (i, r)

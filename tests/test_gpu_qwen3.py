@@ -138,45 +138,36 @@ def test_cpp_model_mirror(models, pkg, synth, tmp_path):
         assert abs(float(cs) - float(lg.astype(np.float64).sum())) <= 1e-3 * max(1.0, float(np.abs(lg).sum()))
 
 
-def _logits_in_child(tmp_path, env, passes):
-    """Logits of each pass of a fresh TINY model in a child process started with `env` set."""
-    import subprocess
-    import sys
-
-    out = tmp_path / "child.npy"
-    code = (
-        "import sys, numpy as np\n"
-        f"sys.path.insert(0, {os.path.dirname(os.path.dirname(os.path.abspath(__file__)))!r})\n"
-        "from __graft_entry__ import import_package\n"
-        "from oracle import ora\n"
-        "from tests.qwen3_fixture import TINY, build\n"
-        "pkg = import_package()\n"
-        "m = pkg.Qwen3Model(**TINY)\n"
-        "build(pkg.synth, ora, TINY, 900, gpu_model=m)\n"
-        f"np.save({str(out)!r}, np.stack([m.forward(ids) for ids in {passes!r}]))\n")
-    subprocess.run([sys.executable, "-c", code], check=True, env=dict(os.environ, **env), timeout=100)
-    return np.load(out)
+def _logits_with_option(gpu, option, value, passes):
+    """Logits of each pass on the same model with one test switch of a81w41_qwen3_set_option on."""
+    gpu.set_option(option, value)
+    try:
+        gpu.reset()
+        return np.stack([gpu.forward(ids) for ids in passes])
+    finally:
+        gpu.set_option(option, 0)
+        gpu.reset()
 
 
-def test_fused_prefill_is_bit_identical_to_separate_kernels(models, tmp_path):
+def test_fused_prefill_is_bit_identical_to_separate_kernels(models):
     """With several rows the norms and SiLU*mul write quantised blocks directly; the blocks, and so the
-    logits, must be the very bits of the separate norm / SiLU -> quantiser -> GEMM sequence, which a
-    child process runs with the fusion switched off."""
+    logits, must be the very bits of the separate norm / SiLU -> quantiser -> GEMM sequence, which the
+    same model runs with the fusion switched off."""
     gpu, _ = models
     ids = [(53 * i + 7) % TINY["vocab"] for i in range(23)]
     gpu.reset()
     fused = gpu.forward(ids)
-    assert np.array_equal(fused, _logits_in_child(tmp_path, {"A81W41_QWEN3_UNFUSED": "1"}, [ids])[0])
+    assert np.array_equal(fused, _logits_with_option(gpu, "unfused", 1, [ids])[0])
 
 
-def test_attention_quantised_output_is_bit_identical(models, tmp_path):
-    """For one token the attention kernel writes o_proj's input as quantised blocks; a child process
+def test_attention_quantised_output_is_bit_identical(models):
+    """For one token the attention kernel writes o_proj's input as quantised blocks; with the switch on it
     writes fp32 and lets o_proj quantise it.  Same bits in, so same logits out, step after step."""
     gpu, _ = models
     passes = [[5, 6, 7, 300, 12, 99, 41], [17], [230], [8], [8]]
     gpu.reset()
     here = np.stack([gpu.forward(ids) for ids in passes])
-    assert np.array_equal(here, _logits_in_child(tmp_path, {"A81W41_QWEN3_ATTN_FP32": "1"}, passes))
+    assert np.array_equal(here, _logits_with_option(gpu, "attn_fp32", 1, passes))
 
 
 def test_long_prompt_in_two_chunks(pkg, synth, ora):
@@ -192,25 +183,25 @@ def test_long_prompt_in_two_chunks(pkg, synth, ora):
     assert rel(gpu.forward([77]), cpu.forward([77])) <= TOL      # decode on top reads what the chunks cached
 
 
-def test_gate_up_quantised_output_is_bit_identical(models, tmp_path):
+def test_gate_up_quantised_output_is_bit_identical(models):
     """For one token the gate|up launch writes silu(gate) * up as quantised blocks instead of its fp32
-    outputs; a child process keeps the fp32 outputs and lets down_proj's prologue do it.  Same bits."""
+    outputs; with the switch on it keeps the fp32 outputs and down_proj's prologue does it.  Same bits."""
     gpu, _ = models
     passes = [[9, 450, 3, 3, 27, 81, 200, 11, 64], [100], [101], [7]]
     gpu.reset()
     here = np.stack([gpu.forward(ids) for ids in passes])
-    assert np.array_equal(here, _logits_in_child(tmp_path, {"A81W41_QWEN3_NO_PAIR": "1"}, passes))
+    assert np.array_equal(here, _logits_with_option(gpu, "no_pair", 1, passes))
 
 
-def test_split_attention_for_one_token(models, tmp_path):
-    """The one-token attention with every head's context cut into 4 shares (a child process forces it
-    on this short context): same logits as the single-workgroup kernel up to the grouping of the sums."""
+def test_split_attention_for_one_token(models):
+    """The one-token attention with every head's context cut into 4 shares (forced by the switch on this
+    short context): same logits as the single-workgroup kernel up to the grouping of the sums."""
     gpu, cpu = models
     passes = [[(41 * i + 9) % TINY["vocab"] for i in range(37)], [17], [230], [8], [301]]
     gpu.reset(); cpu.reset()
     here = np.stack([gpu.forward(ids) for ids in passes])
     want = np.stack([cpu.forward(ids) for ids in passes])
-    split = _logits_in_child(tmp_path, {"A81W41_ATTENTION_SPLIT": "4"}, passes)
+    split = _logits_with_option(gpu, "attention_split", 4, passes)
     for a, b, c in zip(split, here, want):
         assert rel(a, c) <= TOL
         assert rel(a, b) <= 1e-3
@@ -256,3 +247,18 @@ def test_full_width_layer_against_the_oracle(pkg, synth, ora):
     errs.append(rel(gpu.forward([1, 2, 3]), cpu.forward([1, 2, 3])))      # a few rows: the few-row kernels
     assert max(errs) <= wide_tol, errs
     assert sorted(errs)[len(errs) // 2] <= TOL, errs                       # and typically within the usual bar
+
+
+@pytest.mark.parametrize("hidden,inter", [(1024, 3072), (2048, 6144)])
+def test_one_token_pass_on_narrow_models(pkg, synth, ora, hidden, inter):
+    """Qwen3-0.6B / 1.7B widths: short activation rows in wide workgroups (hidden 1024 would give the paired
+    gate|up launch sixteen column groups per workgroup, more than its eight-group units allow).  Decode
+    steps against the oracle, and the paired launch against the unpaired one bit for bit."""
+    cfg = dict(n_layers=1, hidden=hidden, n_q_heads=16, n_kv_heads=8, intermediate=inter, vocab=512, max_seq=32)
+    gpu, cpu = pkg.Qwen3Model(**cfg), qf.Qwen3Oracle(**cfg)
+    build(synth, ora, cfg, 921, gpu_model=gpu, oracle_model=cpu)
+    passes = [[3, 99, 500, 7], [17], [230], [8]]
+    here = [gpu.forward(ids) for ids in passes]
+    for got, ids in zip(here, passes):
+        assert rel(got, cpu.forward(ids)) <= 2e-2
+    assert np.array_equal(np.stack(here), _logits_with_option(gpu, "no_pair", 1, passes))

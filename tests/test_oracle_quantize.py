@@ -71,3 +71,30 @@ def test_m_rows_are_independent(ora, synth):
     whole = ora.quantize(x, True).reshape(5, -1)
     for m in range(5):
         assert np.array_equal(whole[m], ora.quantize(x[m], True))
+
+
+@pytest.mark.parametrize("fp32", [False, True])
+def test_overflowing_inverse_scale_gives_the_x86_answer(ora, fp32):
+    """amax < ~3.7e-37: 127/amax = +inf, every x*id is +-inf or (for x = 0) NaN, cvtps_epi32 answers
+    0x80000000 for each of them, the saturating packs make that -128, and the int32 sum of 32 such values
+    wraps to 0 (32 * -2^31 = 0 mod 2^32), so scaled_sum = d * 0 (quantized_gemx_kernels.cc:735-780).  The
+    expected bytes are written out here; tests/test_oracle_avx2.py has the x86 instructions confirm them."""
+    tiny = np.float32(1e-38)
+    x = np.zeros((3, 64), np.float32)
+    x[0, :32] = tiny * np.linspace(-1.0, 1.0, 32, dtype=np.float32)
+    x[0, 5] = 0.0
+    x[0, 32:] = np.float32(1.0)                       # ordinary neighbour in the same super-block
+    x[1, 32:] = 0.0
+    x[1, 32 + 9] = np.float32(-3e-39)                 # subnormal amax, every other element zero
+    x[2, :32] = np.float32(3.8e-37)                   # just above the threshold: finite id, ordinary result
+    x[2, 3] = 0.0
+    q, d, ss = parse_act_blob(ora.quantize(x, fp32), fp32)
+    f = (lambda v: np.float32(v)) if fp32 else (lambda v: np.float32(np.float16(v)))
+    assert (q[0, 0] == -128).all() and ss[0, 0] == 0.0 and d[0, 0] == f(tiny / np.float32(127))
+    assert (q[0, 1] == 127).all()
+    assert (q[1, 1] == -128).all() and ss[1, 1] == 0.0
+    assert not q[1, 0].any() and d[1, 0] == 0.0
+    want = np.full(32, 127, np.int8)
+    want[3] = 0
+    assert np.array_equal(q[2, 0], want)
+    assert ss[2, 0] == f(np.float32(3.8e-37) / np.float32(127) * np.float32(31 * 127))
