@@ -97,6 +97,18 @@ int a81w41_gemv_repack_A81W41_fp16(const void *A_repack_dev, const void *B_repac
 int a81w41_gemm_repack_A81W41_fp32(const void *A_repack_dev, const void *B_repack_dev, float *C_dev,
                                    int M, int N, int K, void *stream);
 
+/* The same contraction for callers that cannot allocate device memory (code under HIP graph
+ * capture from the first call on, tight serving loops, harnesses that forbid it).  No
+ * counterpart in the reference.  Same arguments and the same results bit for bit as
+ * a81w41_gemm_repack_A81W41_fp32; never calls hipMalloc / hipFree.  The partial tiles of the K
+ * split go to a file-scope device array of the library: 2048 tiles = 32 MiB plus 8 KiB of
+ * counters, held by every GPU the library runs on from load to process end.  A shape whose
+ * schedule parks more partial tiles than that (on a 256-CU device only launches of 683 .. 767
+ * tiles of 64 x 64 over K >= 12288, e.g. M = 700 on 12288 -> 4096) is rejected with A81W41_ERR_INVALID_ARG.  All calls
+ * on one GPU share the array, whatever their streams: calls that overlap in time race. */
+int a81w41_gemm_repack_A81W41_fp32_static(const void *A_repack_dev, const void *B_repack_dev,
+                                          float *C_dev, int M, int N, int K, void *stream);
+
 /* Test hook, host only (no device is touched): walks the work list the M > 8 kernels would be
  * launched with for an M x N x K call on a device that holds `resident_workgroups` of them on
  * `cus` compute units (tile = 2: 64 x 64 tiles, 1: 32 x 128 tiles).  Returns the number of

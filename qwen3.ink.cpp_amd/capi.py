@@ -27,6 +27,7 @@ SIGNATURES = {
     "a81w41_quantize_row_q8_1_repack_fp32": (_i, [_vp, _vp, _i64, _vp]),
     "a81w41_gemv_repack_A81W41_fp16": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "a81w41_gemm_repack_A81W41_fp32": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "a81w41_gemm_repack_A81W41_fp32_static": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "a81w41_gemm_schedule_selfcheck": (_i, [_i, _i, _i, _i, _i, _i]),
     "a81w41_block_idot": (_i, [_vp, _i, _vp, _i, _vp, _i, _i, _i, _vp]),
     "a81w41_repack_w80_weight": (_i, [_i, _i, _i, _vp, _vp, _vp]),

@@ -76,8 +76,12 @@ void gemm_scratch_destroy(GemmScratch* ws);
 // The scratch that belongs to stream s on the current device, created at the first call for that stream
 // (which therefore must not come while s is being captured: hipErrorStreamCaptureUnsupported).
 hipError_t gemm_scratch_for_stream(hipStream_t s, GemmScratch* out);
+// The current device's copy of the library's file-scope scratch array (nothing is allocated).
+hipError_t gemm_static_scratch(GemmScratch* out);
+int gemm_static_scratch_tiles();
 // Partial tiles the schedule of an M x N x K call parks (0: no K split); -1 if the device cannot be queried.
 int gemm_partial_tiles(int M, int N, int K);
+hipError_t clear_gemm_counters(const GemmScratch& ws, hipStream_t s);
 // hipErrorInvalidValue if the call's schedule needs more partial tiles than ws holds.
 hipError_t launch_gemm_fp32(const void* A, const void* B, float* C, int M, int N, int K, const GemmScratch& ws, hipStream_t s);
 // Walks the work list of a launch on the host (wm = 1: 32 x 128 tiles, 2: 64 x 64) for a device with

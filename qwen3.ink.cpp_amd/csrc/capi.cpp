@@ -290,7 +290,7 @@ static int stream_scratch(void* stream, int M, int N, int K, a81w41::GemmScratch
     if (e == hipErrorStreamCaptureUnsupported)
         return fail(A81W41_ERR_INVALID_ARG,
                     "the first K-split GEMM call on a stream allocates that stream's scratch and cannot be captured: "
-                    "call once before the capture or use a layer object");
+                    "call once before the capture, use a layer object, or a81w41_gemm_repack_A81W41_fp32_static");
     if (e == hipErrorOutOfMemory) return fail(A81W41_ERR_HIP, "GEMM scratch: out of device memory or more than 16 streams");
     if (e != hipSuccess) return hip_fail(e, "gemm_scratch_for_stream");
     return A81W41_OK;
@@ -323,6 +323,25 @@ int a81w41_gemm_repack_A81W41_fp32(const void* A_repack_dev, const void* B_repac
         return fail(A81W41_ERR_INVALID_ARG, "activation blob must be 16-byte aligned");
     a81w41::GemmScratch ws;
     if (int st = stream_scratch(stream, M, N, K, &ws)) return st;
+    HIP_TRY(a81w41::launch_gemm_fp32(A_repack_dev, B_repack_dev, C_dev, M, N, K, ws, static_cast<hipStream_t>(stream)));
+    return A81W41_OK;
+}
+
+int a81w41_gemm_repack_A81W41_fp32_static(const void* A_repack_dev, const void* B_repack_dev, float* C_dev, int M,
+                                          int N, int K, void* stream) {
+    if (int st = contract_args_ok(A_repack_dev, B_repack_dev, C_dev, M, N, K)) return st;
+    if (reinterpret_cast<uintptr_t>(A_repack_dev) & 15)
+        return fail(A81W41_ERR_INVALID_ARG, "activation blob must be 16-byte aligned");
+    const int need = a81w41::gemm_partial_tiles(M, N, K);
+    if (need < 0) return fail(A81W41_ERR_HIP, "cannot query the device");
+    if (need > a81w41::gemm_static_scratch_tiles())
+        return fail(A81W41_ERR_INVALID_ARG,
+                    "M=%d N=%d K=%d parks %d partial tiles, the static scratch holds %d: use a81w41_gemm_repack_A81W41_fp32",
+                    M, N, K, need, a81w41::gemm_static_scratch_tiles());
+    a81w41::GemmScratch ws;
+    HIP_TRY(a81w41::gemm_static_scratch(&ws));
+    // the array keeps what the last call left: the counters must start at zero
+    if (need > 0) HIP_TRY(a81w41::clear_gemm_counters(ws, static_cast<hipStream_t>(stream)));
     HIP_TRY(a81w41::launch_gemm_fp32(A_repack_dev, B_repack_dev, C_dev, M, N, K, ws, static_cast<hipStream_t>(stream)));
     return A81W41_OK;
 }

@@ -443,14 +443,25 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
 // A scratch is `max_partials` partial tiles of kPartialWords floats plus as many arrival counters, which
 // are zero between launches.  Launches that share a scratch must not overlap in time, so every owner
 // has its own: a context (all of its layers' calls), a stream (the free-standing GEMM entry point: calls
-// on one stream are ordered by the stream, calls on different streams get different scratches).
+// on one stream are ordered by the stream, calls on different streams get different scratches), or the
+// file-scope array below for the entry point that may not allocate.
 constexpr int kMaxPartials = 4096;  // room for every tile of a launch that does not fill the chip to be cut in four
 constexpr int kMaxDevices = 64;
 constexpr int kMaxStreamsPerDevice = 16;
 
+// Static scratch of the allocation-free entry point: 2048 partial tiles (32 MiB) and their counters per
+// device, held from the moment the code object is loaded until the process ends.
+constexpr int kStaticPartials = 2048;
+struct __align__(256) StaticScratch {
+    float partials[(size_t)kStaticPartials * kPartialWords];
+    unsigned arrivals[kStaticPartials];
+};
+static __device__ __align__(256) StaticScratch scratch;
+
 struct DeviceInfo {
     int slots = 0;  // workgroups of the tile kernels the device holds at once (four per CU)
     int cus = 0;
+    StaticScratch* static_scratch = nullptr;  // this device's copy of `scratch`
     struct {
         hipStream_t stream;
         GemmScratch ws;
@@ -485,6 +496,11 @@ hipError_t device_info_locked(DeviceInfo*& out) {
     }
     out = &d;
     return hipSuccess;
+}
+
+__global__ void clear_counters_kernel(unsigned* p, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
 }
 
 // The schedule of one launch (see Schedule): a pure function of the shape and of the device's size.
@@ -645,6 +661,27 @@ hipError_t gemm_scratch_for_stream(hipStream_t s, GemmScratch* out) {
     return hipSuccess;
 }
 
+hipError_t gemm_static_scratch(GemmScratch* out) {
+    std::lock_guard<std::mutex> lock(g_dev_mutex);
+    DeviceInfo* d = nullptr;
+    hipError_t e = device_info_locked(d);
+    if (e != hipSuccess) return e;
+    if (d->static_scratch == nullptr) {
+        // `scratch` names the array for the host compiler only; its address on the current device comes from here
+        StaticScratch* ptr = nullptr;
+        e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (ptr == nullptr) return hipErrorInvalidSymbol;
+        d->static_scratch = ptr;
+    }
+    out->partials = d->static_scratch->partials;
+    out->arrivals = d->static_scratch->arrivals;
+    out->max_partials = kStaticPartials;
+    return hipSuccess;
+}
+
+int gemm_static_scratch_tiles() { return kStaticPartials; }
+
 int gemm_partial_tiles(int M, int N, int K) {
     const int kernel = pick_kernel(M, N, K);
     if (kernel == 0) return 0;
@@ -658,6 +695,12 @@ int gemm_partial_tiles(int M, int N, int K) {
     else
         make_schedule<2>(M, N, K, d->slots, d->cus, kMaxPartials, sc, grid);
     return sc.r * sc.c;
+}
+
+hipError_t clear_gemm_counters(const GemmScratch& ws, hipStream_t s) {
+    const int n = ws.max_partials;
+    hipLaunchKernelGGL(clear_counters_kernel, dim3((n + 255) / 256), dim3(256), 0, s, ws.arrivals, n);
+    return hipGetLastError();
 }
 
 hipError_t launch_gemm_fp32(const void* A, const void* B, float* C, int M, int N, int K, const GemmScratch& ws, hipStream_t s) {

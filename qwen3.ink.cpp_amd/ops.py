@@ -88,12 +88,13 @@ def gemv_fp16(a_blob, b_blob, N: int, K: int, M: int = 1, out=None):
     return out
 
 
-def gemm_fp32(a_blob, b_blob, M: int, N: int, K: int, out=None):
-    """gemm_repack_A81W41_fp32; ``b_blob`` is a uint8 CUDA tensor or a raw device address."""
+def gemm_fp32(a_blob, b_blob, M: int, N: int, K: int, out=None, static_scratch: bool = False):
+    """gemm_repack_A81W41_fp32; ``b_blob`` is a uint8 CUDA tensor or a raw device address.
+    ``static_scratch``: the entry point that allocates nothing (``..._fp32_static``)."""
     torch = _torch()
     if out is None:
         out = torch.empty((M, N), dtype=torch.float32, device=a_blob.device)
-    fn = capi.lib().a81w41_gemm_repack_A81W41_fp32
+    fn = capi.lib().a81w41_gemm_repack_A81W41_fp32_static if static_scratch else capi.lib().a81w41_gemm_repack_A81W41_fp32
     capi.check(fn(_dev_ptr(a_blob), _dev_ptr(b_blob), _dev_ptr(out), M, N, K, _stream()))
     return out
 

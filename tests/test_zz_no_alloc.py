@@ -1,0 +1,55 @@
+"""The GEMM entry point that allocates nothing (a81w41_gemm_repack_A81W41_fp32_static): the partial
+tiles of its K split live in a file-scope device array of the library.  Checked through the C ABI
+against the entry point it is a variant of, bit for bit, and against the oracle."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(ora, synth, torch, M, N, K, seed):
+    w4, s, o = synth.weight_files(N, K, seed)
+    x = synth.activations(M, K, seed + 1, outliers=True)
+    ba, bw = ora.quantize(x, True), ora.repack(w4, s, o, K, N, True)
+    return torch.from_numpy(ba).cuda(), torch.from_numpy(bw).cuda(), ora.gemm_fp32(ba, bw, M, N, K)
+
+
+def test_static_scratch_gemm_equals_the_allocating_entry_point(pkg, ora, synth):
+    import torch
+
+    L = pkg.capi.lib()
+    # two calls in a row, the second smaller; then a shape without a K split and a few-row call.
+    # (322, 1024, 4096) and (130, 136, 2048) split K (partial tiles parked in the static array).
+    cases = [(322, 1024, 4096, 401), (130, 136, 2048, 403), (64, 64, 1024, 405), (5, 64, 256, 407), (322, 1024, 4096, 401)]
+    assert L.a81w41_gemm_schedule_selfcheck(322, 1024, 4096, 1024, 256, 2) > 0
+    assert L.a81w41_gemm_schedule_selfcheck(130, 136, 2048, 1024, 256, 2) > 0
+    for M, N, K, seed in cases:
+        a, b, want = _case(ora, synth, torch, M, N, K, seed)
+        ref = pkg.ops.gemm_fp32(a, b, M, N, K)
+        got = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        pkg.ops.gemm_fp32(a, b, M, N, K, out=got, static_scratch=True)
+        torch.cuda.synchronize()
+        assert torch.equal(got, ref), (M, N, K)
+        g = got.cpu().numpy().astype(np.float64)
+        err = np.max(np.linalg.norm(g - want, axis=1) / np.linalg.norm(want.astype(np.float64), axis=1))
+        assert err <= 1e-4, (M, N, K, err)
+
+
+def test_static_scratch_gemm_rejects_what_does_not_fit(pkg):
+    import torch
+
+    L = pkg.capi.lib()
+    M, N, K = 700, 4096, 12288          # 704 tiles over K = 12288: cut in four = 2816 partial tiles > 2048
+    assert L.a81w41_gemm_schedule_selfcheck(M, N, K, 1024, 256, 2) > 2048
+    a = torch.zeros(M * (K // 64) * 80, dtype=torch.uint8, device="cuda")
+    b = torch.zeros((N // 8) * (K // 64) * 384, dtype=torch.uint8, device="cuda")
+    c = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    st = L.a81w41_gemm_repack_A81W41_fp32_static(C.c_void_p(a.data_ptr()), C.c_void_p(b.data_ptr()), C.c_void_p(c.data_ptr()),
+                                                 M, N, K, None)
+    assert st == 1 and b"static scratch" in L.a81w41_last_error()
+    # the allocating entry point takes the same call
+    pkg.ops.gemm_fp32(a, b, M, N, K, out=c)
+    torch.cuda.synchronize()
+    assert float(c.abs().max()) == 0.0
