@@ -274,6 +274,20 @@ enum {
     A81W41_QWEN3_OPT_ATTENTION_SPLIT = 4   /* value 1..16: shares per head of the one-token attention; 0: automatic */
 };
 int a81w41_qwen3_set_option(a81w41_qwen3 *model, int option, int value);
+/* Parity hook: copies the first `count` floats of one of the model's activation buffers to the host
+ * after the work enqueued so far has finished.  After a pass the buffers hold what the LAST layer left
+ * (the fused passes skip some of them: switch A81W41_QWEN3_OPT_UNFUSED on to have every stage written):
+ * RESIDUAL [rows][hidden] the residual stream after the final add, NORMED its final RMSNorm,
+ * QKV [rows][(n_q + 2 n_kv)*128] with q normalised and rotated in place and k, v as projected (their
+ * normalised / rotated / binary16 form is what the cache holds), ATTENTION [rows][n_q*128],
+ * BLOCK_OUT [rows][hidden] the down projection, GATE_UP [rows][2*intermediate], ACT [rows][intermediate]
+ * = silu(gate)*up, LOGITS [vocab] of the last token. */
+enum {
+    A81W41_QWEN3_BUF_RESIDUAL = 0, A81W41_QWEN3_BUF_NORMED = 1, A81W41_QWEN3_BUF_QKV = 2,
+    A81W41_QWEN3_BUF_ATTENTION = 3, A81W41_QWEN3_BUF_BLOCK_OUT = 4, A81W41_QWEN3_BUF_GATE_UP = 5,
+    A81W41_QWEN3_BUF_ACT = 6, A81W41_QWEN3_BUF_LOGITS = 7
+};
+int a81w41_qwen3_read_buffer(a81w41_qwen3 *model, int which, float *host_out, size_t count);
 /* Forget the cached context (position 0). */
 int a81w41_qwen3_reset(a81w41_qwen3 *model);
 /* Qwen3ForCausalLM::forward: n_tokens new token ids (host) on top of the cached context;

@@ -126,6 +126,25 @@ def linear_forward(x: np.ndarray, b16: np.ndarray, b32: np.ndarray, N: int) -> n
     return out
 
 
+def linear_forward_fast(x: np.ndarray, b16: np.ndarray, b32: np.ndarray, N: int, threads: int = 0) -> np.ndarray:
+    """linear_forward through the AVX2+OpenMP port (bit-identical to the scalar functions, see
+    tests/test_oracle_avx2.py): for full-size checks that the scalar oracle would take minutes for."""
+    x = np.ascontiguousarray(x, np.float32)
+    M, K = x.shape
+    L = avx()
+    threads = threads or L.avx_max_threads()
+    out = np.zeros((M, N), dtype=np.float32)
+    if M > 1:
+        a = np.zeros(M * K // 64 * 80, dtype=np.uint8)
+        L.avx_quantize_row_q8_1_repack_fp32(_p(x), _p(a), x.size)
+        L.avx_gemm_repack_A81W41_fp32(_p(a), _p(b32), _p(out), M, N, K, threads)
+    else:
+        a = np.zeros(K // 64 * 72, dtype=np.uint8)
+        L.avx_quantize_row_q8_1_repack_fp16(_p(x), _p(a), x.size)
+        L.avx_gemv_repack_A81W41_fp16(_p(a), _p(b16), _p(out), 1, N, K, threads)
+    return out
+
+
 def quantize_weight_q41(w: np.ndarray):
     w = np.ascontiguousarray(w, np.float32)
     N, K = w.shape

@@ -14,9 +14,12 @@ Follows, in numpy:
   sample_token_greedy            qwen3/src/qwen/Pipeline.cc:54-62          (first maximum)
 Every linear is oracle.ora.linear_forward, the C restatement of the A81W41 layer with the
 reference's dispatch on M.  Deliberate differences from the reference, shared with the GPU
-build: the KV cache holds IEEE binary16 values (the reference's holds fp32), gate_proj and
-up_proj are one 2*intermediate-wide linear (gate rows first), the cos/sin tables are computed
-here (theta given) instead of loaded from rotary_emb files.
+build: the KV cache holds IEEE binary16 values (the reference's holds fp32, QwenAttention.cc:13-16),
+the embedding table is given as binary16 (the reference's is fp32, ops/embedding.cc:13-26), gate_proj
+and up_proj are one 2*intermediate-wide linear (gate rows first), the cos/sin tables are computed
+here (theta given) instead of loaded from rotary_emb files.  kv_dtype=np.float32 together with an
+fp32 embedding table gives the reference's own storage choices; tests/test_oracle_qwen3.py measures
+what the two narrowings cost at the logits.
 
 Pinned by tests/test_oracle_qwen3.py through properties the mathematics fixes (RMS of a
 normalised row, norm preservation and relative-position property of the rotation, softmax
@@ -68,7 +71,9 @@ def silu_mul(g: np.ndarray, u: np.ndarray) -> np.ndarray:
 
 class Qwen3Oracle:
     def __init__(self, n_layers, hidden, n_q_heads, n_kv_heads, intermediate, vocab, max_seq,
-                 rope_theta=1e6, rms_eps=1e-6):
+                 rope_theta=1e6, rms_eps=1e-6, kv_dtype=np.float16, fast_linear=False):
+        self.kv_dtype = kv_dtype          # np.float32: the reference's cache
+        self.fast_linear = fast_linear    # linears through the AVX2 port (same bits, for full-size models)
         self.L, self.H, self.nq, self.nkv, self.I, self.V, self.S = n_layers, hidden, n_q_heads, n_kv_heads, intermediate, vocab, max_seq
         self.eps = rms_eps
         self.cos, self.sin = rope_tables(max_seq, rope_theta)
@@ -81,15 +86,15 @@ class Qwen3Oracle:
 
     def reset(self):
         self.pos = 0
-        self.k = np.zeros((self.L, self.nkv, self.S, HEAD_DIM), np.float16)
-        self.v = np.zeros((self.L, self.nkv, self.S, HEAD_DIM), np.float16)
+        self.k = np.zeros((self.L, self.nkv, self.S, HEAD_DIM), self.kv_dtype)
+        self.v = np.zeros((self.L, self.nkv, self.S, HEAD_DIM), self.kv_dtype)
 
     def _linear(self, x, entry):
         b16, b32, N = entry
         if b32 is None:
             b32 = np.zeros(1, np.uint8)   # never read: only M == 1 calls go here
             assert x.shape[0] == 1
-        return ora.linear_forward(x, b16, b32, N)
+        return (ora.linear_forward_fast if self.fast_linear else ora.linear_forward)(x, b16, b32, N)
 
     def forward(self, ids) -> np.ndarray:
         ids = np.asarray(ids, np.int64)
@@ -110,8 +115,8 @@ class Qwen3Oracle:
             cos, sin = self.cos[p0:p0 + M, None, :], self.sin[p0:p0 + M, None, :]
             q = rotate_half_apply(q, cos, sin)
             k = rotate_half_apply(k, cos, sin)
-            self.k[l][:, p0:p0 + M] = k.transpose(1, 0, 2).astype(np.float16)
-            self.v[l][:, p0:p0 + M] = v.transpose(1, 0, 2).astype(np.float16)
+            self.k[l][:, p0:p0 + M] = k.transpose(1, 0, 2).astype(self.kv_dtype)
+            self.v[l][:, p0:p0 + M] = v.transpose(1, 0, 2).astype(self.kv_dtype)
             attn = np.zeros((M, self.nq, HEAD_DIM), np.float32)
             for hq in range(self.nq):
                 K = self.k[l][hq // group, :p0 + M].astype(np.float64)   # [T][128]

@@ -59,6 +59,7 @@ SIGNATURES = {
     "a81w41_qwen3_set_norm": (_i, [_vp, _i, _i, _vp]),
     "a81w41_qwen3_set_embedding": (_i, [_vp, _vp]),
     "a81w41_qwen3_set_option": (_i, [_vp, _i, _i]),
+    "a81w41_qwen3_read_buffer": (_i, [_vp, _i, _vp, _sz]),
     "a81w41_qwen3_reset": (_i, [_vp]),
     "a81w41_qwen3_forward": (_i, [_vp, _vp, _i, _vp]),
     "a81w41_qwen3_attention": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, C.c_float, _i, _vp]),

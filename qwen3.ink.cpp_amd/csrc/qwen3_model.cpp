@@ -443,6 +443,29 @@ int a81w41_qwen3_set_option(a81w41_qwen3* m, int option, int value) {
     return A81W41_OK;
 }
 
+int a81w41_qwen3_read_buffer(a81w41_qwen3* m, int which, float* host_out, size_t count) {
+    if (!m || !host_out) return fail(A81W41_ERR_INVALID_ARG, "null argument");
+    const a81w41_qwen3_config& c = m->cfg;
+    const size_t rows = c.max_seq;
+    const float* src = nullptr;
+    size_t have = 0;
+    switch (which) {
+        case A81W41_QWEN3_BUF_RESIDUAL: src = m->x; have = rows * c.hidden; break;
+        case A81W41_QWEN3_BUF_NORMED: src = m->h; have = rows * c.hidden; break;
+        case A81W41_QWEN3_BUF_QKV: src = m->qkv; have = rows * m->qkv_dim(); break;
+        case A81W41_QWEN3_BUF_ATTENTION: src = m->attn; have = rows * c.n_q_heads * kHeadDim; break;
+        case A81W41_QWEN3_BUF_BLOCK_OUT: src = m->o; have = rows * c.hidden; break;
+        case A81W41_QWEN3_BUF_GATE_UP: src = m->gate_up; have = rows * 2 * c.intermediate; break;
+        case A81W41_QWEN3_BUF_ACT: src = m->act; have = rows * c.intermediate; break;
+        case A81W41_QWEN3_BUF_LOGITS: src = m->logits; have = c.vocab; break;
+        default: return fail(A81W41_ERR_INVALID_ARG, "unknown buffer %d", which);
+    }
+    if (count > have) return fail(A81W41_ERR_INVALID_ARG, "buffer %d holds %zu floats, %zu asked for", which, have, count);
+    Q_HIP(hipStreamSynchronize(m->stream));
+    Q_HIP(hipMemcpy(host_out, src, count * sizeof(float), hipMemcpyDeviceToHost));
+    return A81W41_OK;
+}
+
 int a81w41_qwen3_reset(a81w41_qwen3* m) {
     if (!m) return fail(A81W41_ERR_INVALID_ARG, "null model");
     Q_HIP(hipStreamSynchronize(m->stream));
@@ -529,11 +552,20 @@ int a81w41_qwen3_generate_greedy(a81w41_qwen3* m, const int* prompt, int n_promp
         return fail(A81W41_ERR_INVALID_ARG, "prompt of %d and %d new tokens on top of %d do not fit max_seq %d", n_prompt,
                     n_new, m->host_pos, m->cfg.max_seq);
     hipStream_t s = m->stream;
-    hipEvent_t e0, e1, e2, e3;
-    Q_HIP(hipEventCreate(&e0));
-    Q_HIP(hipEventCreate(&e1));
-    Q_HIP(hipEventCreate(&e2));
-    Q_HIP(hipEventCreate(&e3));
+    // events and graph objects are released on every way out of this function
+    struct Scoped {
+        hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
+        hipGraph_t graph = nullptr;
+        hipGraphExec_t exec = nullptr;
+        ~Scoped() {
+            for (hipEvent_t e : ev)
+                if (e) (void)hipEventDestroy(e);
+            if (exec) (void)hipGraphExecDestroy(exec);
+            if (graph) (void)hipGraphDestroy(graph);
+        }
+    } own;
+    for (hipEvent_t& e : own.ev) Q_HIP(hipEventCreate(&e));
+    const hipEvent_t e0 = own.ev[0], e1 = own.ev[1], e2 = own.ev[2], e3 = own.ev[3];
     Q_HIP(hipMemcpy(m->ids, prompt, (size_t)n_prompt * sizeof(int), hipMemcpyHostToDevice));
     Q_HIP(hipMemset(m->step, 0, sizeof(int)));
     Q_HIP(hipEventRecord(e0, s));
@@ -548,8 +580,8 @@ int a81w41_qwen3_generate_greedy(a81w41_qwen3* m, const int* prompt, int n_promp
     const int n_steps = n_new - 1;
     if (n_steps > 0) {
         // one decode step = a pass over the single id in ids[0] + argmax; captured once, replayed
-        hipGraph_t graph = nullptr;
-        hipGraphExec_t exec = nullptr;
+        hipGraph_t& graph = own.graph;
+        hipGraphExec_t& exec = own.exec;
         bool captured = false;
         if (hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal) == hipSuccess) {
             int st = enqueue_pass(m, 1, s);
@@ -571,8 +603,6 @@ int a81w41_qwen3_generate_greedy(a81w41_qwen3* m, const int* prompt, int n_promp
         }
         Q_HIP(hipEventRecord(e2, s));
         Q_HIP(hipStreamSynchronize(s));
-        if (exec) (void)hipGraphExecDestroy(exec);
-        if (graph) (void)hipGraphDestroy(graph);
         m->host_pos += n_steps;
     } else {
         Q_HIP(hipEventRecord(e2, s));
@@ -583,10 +613,6 @@ int a81w41_qwen3_generate_greedy(a81w41_qwen3* m, const int* prompt, int n_promp
     if (n_steps > 0) Q_HIP(hipEventElapsedTime(&ms12, e3, e2));
     if (prefill_ms) *prefill_ms = ms01;
     if (decode_ms) *decode_ms = ms12;
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
-    (void)hipEventDestroy(e2);
-    (void)hipEventDestroy(e3);
     Q_HIP(hipMemcpy(out_tokens, m->history, (size_t)n_new * sizeof(int), hipMemcpyDeviceToHost));
     return A81W41_OK;
 }

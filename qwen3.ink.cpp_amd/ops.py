@@ -365,6 +365,14 @@ class Qwen3Model:
         """Test switch of ``a81w41_qwen3_set_option`` (see include/a81w41.h)."""
         capi.check(capi.lib().a81w41_qwen3_set_option(self.handle, self.OPTIONS[name], int(value)))
 
+    BUFFERS = {"residual": 0, "normed": 1, "qkv": 2, "attention": 3, "block_out": 4, "gate_up": 5, "act": 6, "logits": 7}
+
+    def read_buffer(self, name: str, rows: int, cols: int) -> np.ndarray:
+        """Parity hook ``a81w41_qwen3_read_buffer``: the first rows x cols floats of an activation buffer."""
+        out = np.empty((rows, cols), np.float32)
+        capi.check(capi.lib().a81w41_qwen3_read_buffer(self.handle, self.BUFFERS[name], out.ctypes.data, out.size))
+        return out
+
     def reset(self):
         capi.check(capi.lib().a81w41_qwen3_reset(self.handle))
 

@@ -126,3 +126,29 @@ def test_full_width_logits_are_sensitive_to_1e_5_in_the_attention(synth, ora, mo
     assert max(errs) > 1e-4, errs          # far more than the 1e-5 that went in
     assert max(errs) < 2e-2, errs
 
+
+
+def test_cost_of_the_fp16_cache_and_embedding(synth, ora, capsys):
+    """The build keeps the KV cache and the embedding table in binary16; the reference keeps both in
+    fp32 (QwenAttention.cc:13-16, ops/embedding.cc:13-26).  The oracle in the reference's storage mode
+    against the oracle in the build's: what the two narrowings move at the logits (tiny model, prompt and
+    decode steps).  The fast (AVX2 port) linears give the same logits as the scalar ones, bit for bit."""
+    def make(kv_dtype, emb_fp32, fast=False):
+        m = qf.Qwen3Oracle(**TINY, kv_dtype=kv_dtype, fast_linear=fast)
+        build(synth, ora, TINY, 900, oracle_model=m)
+        # one fp32 table for both: the build's mode sees it rounded to binary16
+        table = (np.float32(1.0) + synth.standard_normal(TINY["vocab"] * TINY["hidden"], 31)).reshape(
+            TINY["vocab"], TINY["hidden"]).astype(np.float32)
+        m.embedding = table if emb_fp32 else table.astype(np.float16)
+        return m
+
+    ours, ref, fast = make(np.float16, False), make(np.float32, True), make(np.float16, False, fast=True)
+    passes = [[3, 99, 500, 7, 7, 123, 45, 256, 31, 8, 301], [17], [400], [5]]
+    worst = 0.0
+    for ids in passes:
+        a, b, c = ours.forward(ids), ref.forward(ids), fast.forward(ids)
+        assert np.array_equal(a, c)
+        worst = max(worst, float(np.linalg.norm(a - b) / np.linalg.norm(b)))
+    with capsys.disabled():
+        print(f"\n[fp16 KV cache + fp16 embedding vs fp32 storage: logits move by at most {worst:.2e} of their norm]")
+    assert 0.0 < worst <= 2e-2
