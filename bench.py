@@ -73,7 +73,7 @@ def parse():
                     help="only the decode step as one dependent chain, the per-shape GEMV leg and the M=322 GEMM leg "
                          "(no branches, grouped, M-sweep, end-to-end or CPU legs): the launch mix the rocprofv3 "
                          "summaries under profiles/ are taken from")
-    ap.add_argument("--branches", type=int, default=4,
+    ap.add_argument("--branches", type=int, default=8,
                     help="parallel branches the step's independent launches are captured into (1 = one chain)")
     ap.add_argument("--e2e-only", action="store_true", help="run only the end-to-end leg (prints its JSON object)")
     ap.add_argument("--no-m-sweep", action="store_true", help="skip the M sweep on the gate and down shapes")
@@ -350,27 +350,39 @@ def main():
         M = args.gemm_m
 
         def time_forward(shape_name, M, K, N, seed):
+            """(GEMM launch alone, quantiser + GEMM as forward runs them): microseconds per call, each leg
+            captured into a HIP graph of 36 calls (one per layer's weights) so that the host's launch cost
+            is not what is timed."""
             group = [d[shape_name] for d in layers]
             x = torch.from_numpy(synth.activations(M, K, seed, outliers=True)).cuda()
             y = torch.empty((M, N), dtype=torch.float32, device="cuda")
             a_blob = ops.quantize(x, fp32=True)
-            for l in group[:2]:
-                ops.gemm_fp32(a_blob, l.weight_fp32_ptr, M, N, K, out=y)
-                l.forward(x, out=y)
-            stream.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(stream)
-            for l in group:
-                ops.gemm_fp32(a_blob, l.weight_fp32_ptr, M, N, K, out=y)
-            e1.record(stream)
-            stream.synchronize()
-            us = e0.elapsed_time(e1) * 1e3 / len(group)
-            e0.record(stream)
-            for l in group:      # quantiser + GEMM as the layer's forward runs them
-                l.forward(x, out=y)
-            e1.record(stream)
-            stream.synchronize()
-            return us, e0.elapsed_time(e1) * 1e3 / len(group)
+
+            def gemm_only():
+                for l in group:
+                    ops.gemm_fp32(a_blob, l.weight_fp32_ptr, M, N, K, out=y)
+
+            def forward():
+                for l in group:
+                    l.forward(x, out=y)
+
+            out = []
+            for fn in (gemm_only, forward):
+                fn()
+                stream.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=stream):
+                    fn()
+                g.replay()
+                reps = 3
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for _ in range(reps):
+                    g.replay()
+                e1.record(stream)
+                stream.synchronize()
+                out.append(e0.elapsed_time(e1) * 1e3 / (reps * len(group)))
+            return out[0], out[1]
 
         rows = []
         tot_ops, tot_t, tot_tg = 0.0, 0.0, 0.0
@@ -391,8 +403,8 @@ def main():
                  "frac": round(tot_ops / tot_t / 1e6 / INT8_PEAK_TOPS, 4),
                  "gemm_only_TOPS": round(tot_ops / tot_tg / 1e6, 2),
                  "note": "TOPS = 2*M*N*K / forward_us: activation quantiser launch + GEMM launch, per call, weights "
-                         "rotated over the 36 layers' resident copies; gemm_us is the GEMM launch alone on a "
-                         "quantised blob",
+                         "rotated over the 36 layers' resident copies, 36 calls per HIP-graph replay; gemm_us is the "
+                         "GEMM launch alone on a quantised blob",
                  "per_shape": rows,
                  "reference_bench_point_320x12288x4096": {
                      "forward_us": round(fwd320, 2), "gemm_us": round(us320, 2),
@@ -410,15 +422,24 @@ def main():
                 for M in (1, 8, 32, 128, 512, 2048):
                     x = torch.from_numpy(synth.activations(M, K, 96)).cuda()
                     y = torch.empty((M, N), dtype=torch.float32, device="cuda")
-                    group[0].forward(x, out=y)
+
+                    def sweep():
+                        for l in group:
+                            l.forward(x, out=y)
+
+                    sweep()
                     stream.synchronize()
+                    g = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(g, stream=stream):
+                        sweep()
+                    g.replay()
                     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                     e0.record(stream)
-                    for l in group:
-                        l.forward(x, out=y)
+                    g.replay()
+                    g.replay()
                     e1.record(stream)
                     stream.synchronize()
-                    us = e0.elapsed_time(e1) * 1e3 / len(group)
+                    us = e0.elapsed_time(e1) * 1e3 / (2 * len(group))
                     wbytes = (0.625 if M == 1 else 0.75) * K * N
                     m_sweep.append({"shape": name, "M": M, "path": "gemv" if M == 1 else "quantiser + gemm",
                                     "forward_us": round(us, 2), "TOPS": round(2.0 * M * N * K / us / 1e6, 2),

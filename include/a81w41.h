@@ -117,6 +117,11 @@ int a81w41_gemm_repack_A81W41_fp32_static(const void *A_repack_dev, const void *
  * code names the violated property. */
 int a81w41_gemm_schedule_selfcheck(int M, int N, int K, int resident_workgroups, int cus, int tile);
 
+/* Test hook, host only: the same for the layer object's M > 32 kernel (128 x 128 tiles, the (tile,
+ * 32-block) units of a launch cut into equal contiguous runs): every unit exactly once, contributor
+ * ranges and partial-tile slots consistent.  Returns the number of tiles shared between workgroups. */
+int a81w41_gemm_fp6_plan_selfcheck(int M, int N, int K, int resident_workgroups);
+
 /* The int32 block dots both kernels form before scaling (iacc_low / iacc_high,
  * quantized_gemx_kernels.cc:161-168 and :430-457), exposed for parity checks:
  * out_dev[(m*N + n)*(K/32) + 2*sb + h], h = 0 low / 1 high 32-block.
@@ -204,6 +209,16 @@ const void *a81w41_linear_weight_fp32_dev(const a81w41_linear *layer);
  * dispatch -- M == 1: fp16-parameter quantiser + GEMV on the 320 B blob,
  * M > 1: fp32-parameter quantiser + GEMM on the 384 B blob.  Device pointers. */
 int a81w41_linear_forward(a81w41_linear *layer, const float *x_dev, int M, float *y_dev, void *stream);
+/* Which kernel M > 32 calls of this layer contract on.  The layer keeps, beside
+ * the reference's two blobs, its fp32-parameter weights in the operand format of
+ * gfx950's block-scaled matrix op (exact for these integers, twice the int8
+ * rate); by default a call goes there when its shape is one where that kernel is
+ * the faster one (A81W41_KERNEL_AUTO).  The other two values exist for tests and
+ * measurements: NEVER keeps every call on the int8 kernels, ALWAYS sends every
+ * call of more than 32 rows to the block-scaled one.  No counterpart in the
+ * reference, which has one kernel per precision (quantized_gemx_kernels.cc:349). */
+enum { A81W41_KERNEL_AUTO = 0, A81W41_KERNEL_INT8 = 1, A81W41_KERNEL_BLOCK_SCALED = 2 };
+int a81w41_linear_set_kernel(a81w41_linear *layer, int choice);
 /* Several layers applied to the same input in one call: ys_dev[i] = layers[i](x).
  * The reference does this by storing q, k and v as one 4096 -> 6144 layer
  * (QwenAttention.cc:29,78-83) and exports gate_up_proj the same way; here the

@@ -29,6 +29,7 @@ SIGNATURES = {
     "a81w41_gemm_repack_A81W41_fp32": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "a81w41_gemm_repack_A81W41_fp32_static": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "a81w41_gemm_schedule_selfcheck": (_i, [_i, _i, _i, _i, _i, _i]),
+    "a81w41_gemm_fp6_plan_selfcheck": (_i, [_i, _i, _i, _i]),
     "a81w41_block_idot": (_i, [_vp, _i, _vp, _i, _vp, _i, _i, _i, _vp]),
     "a81w41_repack_w80_weight": (_i, [_i, _i, _i, _vp, _vp, _vp]),
     "a81w41_quantize_weight_q40": (_i, [_vp, _i, _i, _vp, _vp]),
@@ -49,6 +50,7 @@ SIGNATURES = {
     "a81w41_linear_weight_fp16_dev": (_vp, [_vp]),
     "a81w41_linear_weight_fp32_dev": (_vp, [_vp]),
     "a81w41_linear_forward": (_i, [_vp, _vp, _i, _vp, _vp]),
+    "a81w41_linear_set_kernel": (_i, [_vp, _i]),
     "a81w41_linear_forward_multi": (_i, [_i, C.POINTER(_vp), _vp, _i, C.POINTER(_vp), _vp]),
     "a81w41_linear_forward_host": (_i, [_vp, _vp, _i, _vp]),
     "a81w41_qwen3_create": (_i, [_vp, C.POINTER(_vp)]),

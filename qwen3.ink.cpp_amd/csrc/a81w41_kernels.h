@@ -88,6 +88,24 @@ hipError_t launch_gemm_fp32(const void* A, const void* B, float* C, int M, int N
 // slots_fit resident workgroups on cus CUs: >= 0 (the partial tiles used) if every tile and chunk is
 // covered exactly once and no partial tile is shared, else a negative code.
 int gemm_schedule_selfcheck(int M, int N, int K, int slots_fit, int cus, int wm);
+// ---- the layer object's M > 32 path: block-scaled fp6 matrix ops on private operand formats (gemm_fp6_a81w41.hip)
+// A6: quantised activations as two 4-bit pieces per value in fp6 patterns, W6: weight codes as fp6 patterns,
+// both with fp32 parameters, in 32-row / 32-column panels.  Rows and columns are padded to multiples of 32.
+constexpr int kGemmFp6MinRows = 33;  // calls with fewer rows stay on the int8 kernels
+// Whether a call of this shape goes to the block-scaled kernel (false: the int8 kernels are as fast or faster).
+bool gemm_fp6_preferred(int M, int N, int K);
+size_t gemm_fp6_a6_bytes(int64_t rows, int K);
+size_t gemm_fp6_w6_bytes(int N, int K);
+hipError_t launch_w384_to_w6(const void* w384, void* w6, int N, int K, hipStream_t s);  // once per layer
+// fp32 rows -> 80 B blocks (y80, may be null: exactly what launch_quantize(fp32) writes) and A6
+hipError_t launch_quantize_a6(const float* x, void* y80, void* a6, int M, int K, hipStream_t s);
+hipError_t launch_a80_to_a6(const void* y80, void* a6, int M, int K, hipStream_t s);  // rows already in 80 B blocks
+// C[M][N]; hipErrorInvalidValue if ws is smaller than a context's scratch
+hipError_t launch_gemm_fp6(const void* a6, const void* w6, float* C, int M, int N, int K, const GemmScratch& ws, hipStream_t s);
+// Host-side walk of a launch's work units for a device holding `slots` workgroups: >= 0 (tiles whose K range is
+// shared between workgroups) if every (tile, block) is covered once and the partial-tile slots are consistent.
+int gemm_fp6_plan_selfcheck(int M, int N, int K, int slots);
+
 // Few-row variant (M <= 8, activation rows resident in LDS, no matrix cores), used by
 // launch_gemm_fp32 when gemm_rows_fits(): same arguments and results within the same tolerance.
 bool gemm_rows_fits(int M, int K);
@@ -109,8 +127,14 @@ hipError_t launch_gemm_a80w40(const void* A, const void* B, float* C, int M, int
 }  // namespace a81w41
 struct a81w41_context;
 namespace a81w41 {
-// The K-split scratch a context owns (capi.cpp).
+// The K-split scratch a context owns, and its A6 scratch (capi.cpp).
 const GemmScratch& context_gemm_scratch(const a81w41_context* ctx);
+void* context_a6_scratch(const a81w41_context* ctx);
+}  // namespace a81w41
+struct a81w41_linear;
+namespace a81w41 {
+const void* linear_w6(const a81w41_linear* layer);  // null if the layer has no fp32-parameter blob
+bool linear_block_scaled(const a81w41_linear* layer, int M);  // an M-row call of this layer contracts on the block-scaled kernel
 
 // Records `message` as the calling thread's last error and returns `status` (capi.cpp).
 int report_failure(int status, const char* message);

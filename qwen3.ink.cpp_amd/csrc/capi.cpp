@@ -132,6 +132,8 @@ struct a81w41_context {
     a81w41::GemmScratch gemm_scratch;  // partial tiles of the GEMM's K split: this context's own
     void* act_scratch = nullptr;  // quantised activations, sized for the fp32 layout
     size_t act_bytes = 0;
+    void* a6_scratch = nullptr;   // the same rows in the M > 32 kernel's operand format
+    size_t a6_bytes = 0;
     int64_t max_elems = 0;
     float* x_stage = nullptr;  // device staging for forward_host
     float* y_stage = nullptr;
@@ -143,10 +145,18 @@ struct a81w41_linear {
     int N = 0, K = 0;
     void* w16 = nullptr;  // device, 320 B blocks
     void* w32 = nullptr;  // device, 384 B blocks
+    void* w6 = nullptr;   // device, the block-scaled kernel's operand format, derived from w32
+    int kernel_choice = A81W41_KERNEL_AUTO;
 };
 
 namespace a81w41 {
 const GemmScratch& context_gemm_scratch(const a81w41_context* ctx) { return ctx->gemm_scratch; }
+void* context_a6_scratch(const a81w41_context* ctx) { return ctx->a6_scratch; }
+const void* linear_w6(const a81w41_linear* layer) { return layer->w6; }
+bool linear_block_scaled(const a81w41_linear* l, int M) {
+    if (!l->w6 || M < kGemmFp6MinRows || l->kernel_choice == A81W41_KERNEL_INT8) return false;
+    return l->kernel_choice == A81W41_KERNEL_BLOCK_SCALED || gemm_fp6_preferred(M, l->N, l->K);
+}
 // Lets the other translation units of the library leave their message where a81w41_last_error() finds it.
 int report_failure(int status, const char* message) { return fail(status, "%s", message); }
 uint16_t float_to_half_bits(float f) { return f32_to_f16(f); }
@@ -352,6 +362,11 @@ int a81w41_gemm_schedule_selfcheck(int M, int N, int K, int resident_workgroups,
     return a81w41::gemm_schedule_selfcheck(M, N, K, resident_workgroups, cus, tile);
 }
 
+int a81w41_gemm_fp6_plan_selfcheck(int M, int N, int K, int resident_workgroups) {
+    if (M < 1 || !shape_ok(N, K) || resident_workgroups < 1) return fail(A81W41_ERR_INVALID_ARG, "bad arguments") * -100;
+    return a81w41::gemm_fp6_plan_selfcheck(M, N, K, resident_workgroups);
+}
+
 int a81w41_gemv_repack_A80W40(const void* A_repack_dev, const void* B_repack_dev, float* C_dev, int M, int N,
                               int K, void* stream) {
     if (int st = contract_args_ok(A_repack_dev, B_repack_dev, C_dev, M, N, K)) return st;
@@ -413,8 +428,13 @@ int a81w41_context_create(int max_rows, int max_cols, a81w41_context** out) {
     ctx->max_elems = (int64_t)max_rows * max_cols;
     ctx->act_bytes = (size_t)(ctx->max_elems / 64) * a81w41::kABlock32;
     HIP_TRY(a81w41::gemm_scratch_create(&ctx->gemm_scratch));
-    if (hipError_t e = hipMalloc(&ctx->act_scratch, ctx->act_bytes); e != hipSuccess) {
+    // A6 holds 2 B per value, rows padded to a multiple of 32 (calls that use it have more than 32 rows)
+    ctx->a6_bytes = 4 * (size_t)ctx->max_elems;
+    hipError_t e = hipMalloc(&ctx->act_scratch, ctx->act_bytes);
+    if (e == hipSuccess) e = hipMalloc(&ctx->a6_scratch, ctx->a6_bytes);
+    if (e != hipSuccess) {
         a81w41::gemm_scratch_destroy(&ctx->gemm_scratch);
+        (void)hipFree(ctx->act_scratch);
         return hip_fail(e, "hipMalloc(activation scratch)");
     }
     *out = ctx.release();
@@ -425,6 +445,7 @@ void a81w41_context_destroy(a81w41_context* ctx) {
     if (!ctx) return;
     a81w41::gemm_scratch_destroy(&ctx->gemm_scratch);
     (void)hipFree(ctx->act_scratch);
+    (void)hipFree(ctx->a6_scratch);
     (void)hipFree(ctx->x_stage);
     (void)hipFree(ctx->y_stage);
     delete ctx;
@@ -454,10 +475,15 @@ int a81w41_linear_create_from_blobs(a81w41_context* ctx, int N, int K, const voi
         const size_t b = a81w41_weight_blob_bytes(K, N, 1);
         e = hipMalloc(&l->w32, b);
         if (e == hipSuccess) e = hipMemcpy(l->w32, blob_fp32, b, hipMemcpyHostToDevice);
+        // the operand format of the M > 32 kernel, derived on the device once
+        if (e == hipSuccess) e = hipMalloc(&l->w6, a81w41::gemm_fp6_w6_bytes(N, K));
+        if (e == hipSuccess) e = a81w41::launch_w384_to_w6(l->w32, l->w6, N, K, nullptr);
+        if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
     }
     if (e != hipSuccess) {
         (void)hipFree(l->w16);
         (void)hipFree(l->w32);
+        (void)hipFree(l->w6);
         return hip_fail(e, "uploading weight blobs");
     }
     *out = l.release();
@@ -504,6 +530,7 @@ void a81w41_linear_destroy(a81w41_linear* l) {
     if (!l) return;
     (void)hipFree(l->w16);
     (void)hipFree(l->w32);
+    (void)hipFree(l->w6);
     delete l;
 }
 
@@ -522,6 +549,17 @@ int a81w41_linear_forward(a81w41_linear* l, const float* x_dev, int M, float* y_
     // QwenOperator.cc:96-120: the precision of the activation parameters follows M.
     if (M > 1) {
         if (!l->w32) return fail(A81W41_ERR_INVALID_ARG, "layer has no fp32-parameter blob (needed for M > 1)");
+        if (a81w41::linear_block_scaled(l, M)) {
+            // same quantised rows (the scratch still receives the reference's 80 B blocks), contracted by the
+            // block-scaled matrix ops from the private operand formats
+            if ((reinterpret_cast<uintptr_t>(x_dev) & 3) || (reinterpret_cast<uintptr_t>(y_dev) & 3))
+                return fail(A81W41_ERR_INVALID_ARG, "x and y must be 4-byte aligned");
+            if (int st = check_device()) return st;
+            HIP_TRY(a81w41::launch_quantize_a6(x_dev, ctx->act_scratch, ctx->a6_scratch, M, l->K, static_cast<hipStream_t>(stream)));
+            HIP_TRY(a81w41::launch_gemm_fp6(ctx->a6_scratch, l->w6, y_dev, M, l->N, l->K, ctx->gemm_scratch,
+                                            static_cast<hipStream_t>(stream)));
+            return A81W41_OK;
+        }
         if (int st = a81w41_quantize_row_q8_1_repack_fp32(x_dev, ctx->act_scratch, (int64_t)M * l->K, stream)) return st;
         if (int st = contract_args_ok(ctx->act_scratch, l->w32, y_dev, M, l->N, l->K)) return st;
         HIP_TRY(a81w41::launch_gemm_fp32(ctx->act_scratch, l->w32, y_dev, M, l->N, l->K, ctx->gemm_scratch,
@@ -541,6 +579,14 @@ int a81w41_linear_forward(a81w41_linear* l, const float* x_dev, int M, float* y_
     }
     if (int st = a81w41_quantize_row_q8_1_repack_fp16(x_dev, ctx->act_scratch, (int64_t)M * l->K, stream)) return st;
     return a81w41_gemv_repack_A81W41_fp16(ctx->act_scratch, l->w16, y_dev, M, l->N, l->K, stream);
+}
+
+int a81w41_linear_set_kernel(a81w41_linear* l, int choice) {
+    if (!l) return fail(A81W41_ERR_INVALID_ARG, "null layer");
+    if (choice != A81W41_KERNEL_AUTO && choice != A81W41_KERNEL_INT8 && choice != A81W41_KERNEL_BLOCK_SCALED)
+        return fail(A81W41_ERR_INVALID_ARG, "unknown kernel choice %d", choice);
+    l->kernel_choice = choice;
+    return A81W41_OK;
 }
 
 int a81w41_linear_forward_multi(int n, a81w41_linear* const* layers, const float* x_dev, int M,

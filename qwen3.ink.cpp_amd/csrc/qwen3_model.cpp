@@ -126,6 +126,16 @@ int enqueue_pass(a81w41_qwen3* m, int M, hipStream_t s) {
     const bool quant_fused = M > 1 && prefill_fusion_usable(m);
     void* scratch = a81w41_context_activation_scratch_dev(m->ctx);
     const a81w41::GemmScratch& gws = a81w41::context_gemm_scratch(m->ctx);
+    // the contraction of rows that sit in the scratch as 80 B blocks: where the layer picks the block-scaled
+    // kernel, that one takes them in its own operand format
+    auto gemm_from_scratch = [&](a81w41_linear* lin, float* out, int N, int K) -> hipError_t {
+        if (a81w41::linear_block_scaled(lin, M)) {
+            void* a6 = a81w41::context_a6_scratch(m->ctx);
+            if (hipError_t e = a81w41::launch_a80_to_a6(scratch, a6, M, K, s); e != hipSuccess) return e;
+            return a81w41::launch_gemm_fp6(a6, a81w41::linear_w6(lin), out, M, N, K, gws, s);
+        }
+        return a81w41::launch_gemm_fp32(scratch, a81w41_linear_weight_fp32_dev(lin), out, M, N, K, gws, s);
+    };
     const bool attn_blocks = !m->opt_vector_attention && a81w41::attention_prefill_fits(M, c.n_q_heads, c.n_kv_heads);
     for (int l = 0; l < c.n_layers; l++) {
         LayerWeights& L = m->layers[l];
@@ -133,7 +143,7 @@ int enqueue_pass(a81w41_qwen3* m, int M, hipStream_t s) {
         const float* norm_res = pending ? m->x : nullptr;
         if (quant_fused) {
             Q_HIP(a81w41::launch_add_rmsnorm_quant(norm_in, norm_res, L.norm[0], m->x, scratch, M, c.hidden, c.rms_eps, s));
-            Q_HIP(a81w41::launch_gemm_fp32(scratch, a81w41_linear_weight_fp32_dev(L.lin[0]), m->qkv, M, qkv_dim, c.hidden, gws, s));
+            Q_HIP(gemm_from_scratch(L.lin[0], m->qkv, qkv_dim, c.hidden));
         } else {
             Q_HIP(a81w41::launch_add_rmsnorm(norm_in, norm_res, L.norm[0], m->x, m->h, M, c.hidden, c.rms_eps, s));
             Q_TRY(a81w41_linear_forward(L.lin[0], m->h, M, m->qkv, s));
@@ -143,7 +153,7 @@ int enqueue_pass(a81w41_qwen3* m, int M, hipStream_t s) {
         if (quant_fused && attn_blocks) {  // the matrix-core attention hands o_proj its input as quantised blocks
             Q_HIP(a81w41::launch_attention_prefill(m->qkv, qkv_dim, L.k_cache, L.v_cache, m->pos, nullptr, q_dim, M, c.n_q_heads,
                                                    c.n_kv_heads, c.max_seq, scale, s, scratch));
-            Q_HIP(a81w41::launch_gemm_fp32(scratch, a81w41_linear_weight_fp32_dev(L.lin[1]), m->o, M, c.hidden, q_dim, gws, s));
+            Q_HIP(gemm_from_scratch(L.lin[1], m->o, c.hidden, q_dim));
         } else {
             Q_HIP(a81w41::launch_attention(m->qkv, qkv_dim, L.k_cache, L.v_cache, m->pos, m->attn, q_dim, M, c.n_q_heads,
                                            c.n_kv_heads, c.max_seq, scale, s, m->opt_vector_attention ? 1 : 0));
@@ -151,10 +161,9 @@ int enqueue_pass(a81w41_qwen3* m, int M, hipStream_t s) {
         }
         if (quant_fused) {
             Q_HIP(a81w41::launch_add_rmsnorm_quant(m->o, m->x, L.norm[1], m->x, scratch, M, c.hidden, c.rms_eps, s));
-            Q_HIP(a81w41::launch_gemm_fp32(scratch, a81w41_linear_weight_fp32_dev(L.lin[2]), m->gate_up, M, 2 * c.intermediate,
-                                           c.hidden, gws, s));
+            Q_HIP(gemm_from_scratch(L.lin[2], m->gate_up, 2 * c.intermediate, c.hidden));
             Q_HIP(a81w41::launch_silu_mul_quant(m->gate_up, scratch, M, c.intermediate, s));
-            Q_HIP(a81w41::launch_gemm_fp32(scratch, a81w41_linear_weight_fp32_dev(L.lin[3]), m->o, M, c.hidden, c.intermediate, gws, s));
+            Q_HIP(gemm_from_scratch(L.lin[3], m->o, c.hidden, c.intermediate));
         } else {
             Q_HIP(a81w41::launch_add_rmsnorm(m->o, m->x, L.norm[1], m->x, m->h, M, c.hidden, c.rms_eps, s));
             Q_TRY(a81w41_linear_forward(L.lin[2], m->h, M, m->gate_up, s));

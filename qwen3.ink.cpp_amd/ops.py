@@ -268,6 +268,12 @@ class Linear:
         capi.check(capi.lib().a81w41_linear_load(ctx.handle, path.encode(), 1, N, K, C.byref(h)))
         return cls(h, ctx, N, K)
 
+    KERNELS = {"auto": 0, "int8": 1, "block_scaled": 2}
+
+    def set_kernel(self, choice: str) -> None:
+        """Which kernel M > 32 calls contract on: "auto" (by shape, the default), "int8", "block_scaled"."""
+        capi.check(capi.lib().a81w41_linear_set_kernel(self.handle, self.KERNELS[choice]))
+
     def forward(self, x, out=None):
         """x: CUDA float32 [M][K] (or [1][M][K]) -> [M][N]; enqueues on the current stream."""
         torch = _torch()

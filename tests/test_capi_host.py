@@ -91,3 +91,20 @@ def test_gemm_schedule_covers_every_tile_and_chunk_once(pkg, tile):
                 used_split += got > 0
     assert used_split > 20      # the K split really is exercised
     assert L.a81w41_gemm_schedule_selfcheck(0, 64, 64, 1024, 256, 2) < 0   # argument errors are negative too
+
+
+def test_block_scaled_gemm_plan_covers_every_unit_once(pkg):
+    """The layer object's M > 32 kernel cuts the (tile, 32-block) units of a launch into equal contiguous runs:
+    walked on the host for the layer's shapes and odd ones, for several device sizes."""
+    L = pkg.capi.lib()
+    shapes = [(4096, 4096), (4096, 1024), (4096, 12288), (12288, 4096), (4096, 6144), (4096, 24576), (4096, 151936),
+              (512, 256), (4096, 8), (256, 4104), (64, 64), (1024, 40)]
+    shared = 0
+    for K, N in shapes:
+        for M in (33, 64, 65, 128, 129, 322, 512, 640, 1024, 2048, 4096):
+            for slots in (512, 256, 8, 3, 1):
+                got = L.a81w41_gemm_fp6_plan_selfcheck(M, N, K, slots)
+                assert got >= 0, (M, N, K, slots, got)
+                shared += got > 0
+    assert shared > 50
+    assert L.a81w41_gemm_fp6_plan_selfcheck(0, 64, 64, 512) < 0

@@ -90,9 +90,10 @@ def test_prefill_forward_m322(pkg, ora, synth, torch, name):
         assert torch.equal(layer.forward(xd), y)
     # rows are independent: two rows alone (through the same M > 1 path) give the same values;
     # not the same bits, because a few-row call and a split-K tile add the super-blocks in
-    # different groupings
+    # different groupings (and, where the 322-row call runs on the block-scaled kernel, its min
+    # terms carry 16 significant bits)
     two = layer.forward(dev(torch, x[[7, 300]]))
-    assert row_err(two.cpu().numpy(), y[[7, 300]].cpu().numpy()) <= 4e-6
+    assert row_err(two.cpu().numpy(), y[[7, 300]].cpu().numpy()) <= (3e-5 if name in ("gate", "down") else 4e-6)
 
 
 @pytest.mark.parametrize("name,M", [("gate", m) for m in (2, 8, 32, 33, 128, 512, 2048)] +

@@ -403,3 +403,54 @@ def test_gemm_calls_on_two_streams_do_not_share_partial_tiles(pkg, ora, synth, t
         assert torch.equal(alone[i], cases[i][2])
         for r in range(6):
             assert torch.equal(outs[i][r], alone[i]), (i, r)
+
+
+@pytest.mark.parametrize("M,N,K", [(33, 8, 64), (40, 136, 256), (64, 64, 1024), (65, 1000, 2048), (128, 128, 4096),
+                                   (130, 136, 2048), (322, 1024, 4096), (322, 256, 1024), (256, 16384, 256),
+                                   (1030, 4104, 256), (640, 4096, 256), (384, 24576, 512), (100, 512, 12288)])
+def test_layer_forward_block_scaled_kernel(pkg, ora, synth, torch, M, N, K):
+    """The layer object's second M > 32 kernel, on the block-scaled fp6 matrix ops from its own operand
+    formats (by default only for shapes where it is the faster one; forced here): ragged rows and columns
+    (panels padded to 32), one tile shared by many workgroups, many tiles per workgroup, K from one 64-K
+    super-block to 12288.  Same bars as the other kernels; the scratch still receives the reference's 80 B
+    blocks; results repeat bit for bit."""
+    w4, s, o = synth.weight_files(N, K, 601)
+    s = s * np.float32(1.0371)          # fp32 params that fp16 cannot hold
+    x = synth.activations(M, K, 602, outliers=True)
+    ctx = pkg.ops.Context(max_rows=M, max_cols=K)
+    layer = pkg.Linear.from_arrays(w4, s, o, N=N, K=K, ctx=ctx)
+    layer.set_kernel("block_scaled")
+    xd = dev(torch, x)
+    got = layer.forward(xd).cpu().numpy()
+    b16, b32 = ora.repack(w4, s, o, K, N, False), ora.repack(w4, s, o, K, N, True)
+    want = ora.linear_forward_fast(x, b16, b32, N)
+    assert row_err(got, want) <= TOL
+    assert row_err(got, want) <= 3e-5      # the min terms run on 16-bit-significand pieces: below 2^-16 of a term
+    qa = ctx.activation_scratch(M * K // 64 * 80).cpu().numpy()
+    assert not same_bytes(qa, ora.quantize(x, True))
+    assert np.array_equal(layer.forward(xd).cpu().numpy(), got)
+
+
+def test_layer_kernel_choice_at_full_width(pkg, ora, synth, torch):
+    """gate_proj of Qwen3-8B with the 322-row prompt of the reference's benchmark: by default the call runs on the
+    block-scaled kernel (same bits as when forced), the int8 kernel stays selectable, both meet the bar."""
+    M, N, K = 322, 12288, 4096
+    w4, s, o = synth.weight_files(N, K, 611)
+    x = synth.activations(M, K, 612, outliers=True)
+    ctx = pkg.ops.Context(max_rows=M, max_cols=K)
+    layer = pkg.Linear.from_arrays(w4, s, o, N=N, K=K, ctx=ctx)
+    xd = dev(torch, x)
+    auto = layer.forward(xd).cpu().numpy()
+    layer.set_kernel("block_scaled")
+    forced = layer.forward(xd).cpu().numpy()
+    layer.set_kernel("int8")
+    int8 = layer.forward(xd).cpu().numpy()
+    layer.set_kernel("auto")
+    assert np.array_equal(auto, forced)
+    assert not np.array_equal(auto, int8)   # different summation trees
+    b16, b32 = ora.repack(w4, s, o, K, N, False), ora.repack(w4, s, o, K, N, True)
+    want = ora.linear_forward_fast(x, b16, b32, N)
+    assert row_err(int8, want) <= TOL
+    assert row_err(auto, want) <= 3e-5
+    with pytest.raises(Exception):
+        pkg.capi.check(pkg.capi.lib().a81w41_linear_set_kernel(layer.handle, 7))
