@@ -110,6 +110,10 @@ int gemm_fp6_plan_selfcheck(int M, int N, int K, int slots);
 // launch_gemm_fp32 when gemm_rows_fits(): same arguments and results within the same tolerance.
 bool gemm_rows_fits(int M, int K);
 hipError_t launch_gemm_rows_fp32(const void* A, const void* B, float* C, int M, int N, int K, hipStream_t s);
+// 9 <= M <= 32: one row panel, operands loaded straight into registers, K cut inside and between workgroups.
+int gemm_rows32_split(int N, int K);
+hipError_t launch_gemm_rows32_fp32(const void* A, const void* B, float* C, int M, int N, int K, const GemmScratch& ws,
+                                   hipStream_t s);
 // w80: codes count as code - 8 (the A80W40 variant).
 hipError_t launch_block_idot(const void* A, bool a_fp32, const void* B, bool b_fp32, int32_t* out,
                              int M, int N, int K, hipStream_t s, bool w80 = false);

@@ -586,7 +586,8 @@ hipError_t launch_tiles(const void* A, const void* B, float* C, int M, int N, in
     return hipGetLastError();
 }
 
-// Which kernel a call goes to: 0 the few-row kernel (no scratch), 1 the 32 x 128 tiles, 2 the 64 x 64 tiles.
+// Which kernel a call goes to: 0 the few-row kernel (no scratch), 1 the 32 x 128 tiles, 2 the 64 x 64 tiles,
+// 3 the one-row-panel kernel that loads its operands straight into registers (9 .. 32 rows).
 int pick_kernel(int M, int N, int K) {
     // Measurement aids (tuning builds): A81W41_GEMM_TUNE=tile keeps few-row calls on the matrix-core kernels,
     // A81W41_GEMM_TUNE=Tile64 additionally keeps every call on the 64 x 64 arrangement.
@@ -599,6 +600,12 @@ int pick_kernel(int M, int N, int K) {
     // K = 12288) 21.2 against 24.5, N = 4096 and 1024 at K = 4096 equal.
     const int env_n = tuning_env_int("A81W41_GEMM_N32X128");
     const int min_n_32x128 = env_n > 0 ? env_n : 1024;
+    // Narrow layers at 9 .. 32 rows: too few 32 x 128 tiles to go round, so the tile kernels cut K 12- to 16-fold
+    // and the last arriver's merge dominates; the one-row-panel kernel cuts K inside the workgroup instead
+    // (N = 1024, K = 4096: 9.6 against 14.1 us per forward).  From N = 4096 on its per-lane loads of the 80 B
+    // row blocks cost more than the tile kernels' staged copies (gate_proj at 32 rows 32 against 22 us).
+    const int rows32_mode = tuning_env_int("A81W41_GEMM_ROWS32");  // tuning builds: 1 always, 2 never
+    if (M <= 32 && tune != 'T' && rows32_mode != 2 && (N <= 2048 || rows32_mode == 1)) return 3;
     if (M <= 32 && N >= min_n_32x128 && tune != 'T') return 1;
     return 2;
 }
@@ -685,6 +692,10 @@ int gemm_static_scratch_tiles() { return kStaticPartials; }
 int gemm_partial_tiles(int M, int N, int K) {
     const int kernel = pick_kernel(M, N, K);
     if (kernel == 0) return 0;
+    if (kernel == 3) {  // a share of a column panel parks 4 KiB, a quarter of a partial-tile unit
+        const int split = gemm_rows32_split(N, K);
+        return split > 1 ? ((N + 31) / 32 * split + 3) / 4 : 0;
+    }
     std::lock_guard<std::mutex> lock(g_dev_mutex);
     DeviceInfo* d = nullptr;
     if (device_info_locked(d) != hipSuccess) return -1;
@@ -707,6 +718,7 @@ hipError_t launch_gemm_fp32(const void* A, const void* B, float* C, int M, int N
     switch (pick_kernel(M, N, K)) {
         case 0: return launch_gemm_rows_fp32(A, B, C, M, N, K, s);
         case 1: return launch_tiles<1>(A, B, C, M, N, K, ws, s);
+        case 3: return launch_gemm_rows32_fp32(A, B, C, M, N, K, ws, s);
         default: return launch_tiles<2>(A, B, C, M, N, K, ws, s);
     }
 }

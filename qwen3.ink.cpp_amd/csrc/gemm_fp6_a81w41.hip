@@ -38,6 +38,7 @@
 // arrival counter per split tile tells the last contributor to add the parts in contributor order, so the
 // result does not depend on timing.
 #include "a81w41_kernels.h"
+#include "agent_access.h"
 #include "quantize_common.h"
 
 #include <mutex>
@@ -69,23 +70,6 @@ __host__ __device__ __forceinline__ uint32_t split_bf16x2(float x) {
     const uint32_t hi = bf16_rne_bits(x);
     union { uint32_t u; float f; } h = {hi << 16};
     return hi | (bf16_rne_bits(x - h.f) << 16);  // the subtraction is exact
-}
-
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-    __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x0070);  // and lgkmcnt = 0
-}
-// 16-byte accesses at agent scope (served where all XCDs see them, like the 4-byte atomics the compiler would
-// emit, at a quarter of the instructions).  A load's result may be used only after wait_vmcnt<0>().
-typedef float v4f __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ void store16_agent(float* p, v4f v) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
-}
-__device__ __forceinline__ v4f load16_agent(const float* p) {
-    v4f v;
-    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
-    return v;
 }
 
 // ---- operand preparation ------------------------------------------------------------------------
