@@ -421,6 +421,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
                     for (int j = 0; j < 2; j++) sum[i][j] = v16f{0};
                 for (int c = first; c <= last; c++) {
+                    if (c == b) {  // this workgroup's own part is still in registers: the same values it parked
+#pragma unroll
+                        for (int i = 0; i < 2; i++)
+#pragma unroll
+                            for (int j = 0; j < 2; j++) sum[i][j] += acc[i][j];
+                        continue;
+                    }
                     const int cs = run_start(plan, c) >= tile_u0 ? 2 * c : 2 * c + 1;
                     const float* p = partials + (size_t)cs * kTileWords + 4 * tid;
                     v4f l[16];
