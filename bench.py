@@ -440,7 +440,7 @@ def main():
             for name in ("gate", "down"):
                 group = [d[name] for d in layers]     # rotate over the layers' copies: weights from HBM
                 K, N = group[0].K, group[0].N
-                for M in (1, 8, 32, 128, 512, 2048):
+                for M in (1, 8, 32, 128, 512, 2048, 4096):
                     x = torch.from_numpy(synth.activations(M, K, 96)).cuda()
                     y = torch.empty((M, N), dtype=torch.float32, device="cuda")
 
