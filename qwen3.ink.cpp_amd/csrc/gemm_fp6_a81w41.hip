@@ -546,10 +546,14 @@ hipError_t launch_gemm_fp6(const void* a6, const void* w6, float* C, int M, int 
     int slots = 0;
     hipError_t e = resident_workgroups(slots);
     if (e != hipSuccess) return e;
-    const Plan p = make_plan(M, N, K, slots);
     // a run parks at most two partial tiles (its first and its last tile), one counter per run; the scratch is
-    // max_partials units of 16 KiB and as many counters
-    if ((long long)2 * p.grid * kTileWords > (long long)ws.max_partials * 4096 || p.grid > ws.max_partials) return hipErrorInvalidValue;
+    // max_partials units of 16 KiB and as many counters: a device with more CUs than the scratch has room for
+    // gets fewer, longer runs
+    const long long room = (long long)ws.max_partials * 4096 / (2 * kTileWords);
+    if (room < 1) return hipErrorInvalidValue;
+    if (slots > room) slots = (int)room;
+    if (slots > ws.max_partials) slots = ws.max_partials;
+    const Plan p = make_plan(M, N, K, slots);
 #define A81W41_FP6_LAUNCH(ABL)                                                                                              \
     hipLaunchKernelGGL(gemm_a81w41_fp6_kernel<ABL>, dim3(p.grid), dim3(kThreads), 0, s, static_cast<const uint8_t*>(a6), \
                        static_cast<const uint8_t*>(w6), M, N, p.nb, p.tiles_m, p.tiles_n, (M + 31) / 32, (N + 31) / 32, p.units, C, \
