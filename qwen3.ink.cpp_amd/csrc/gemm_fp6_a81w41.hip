@@ -234,10 +234,6 @@ __device__ __forceinline__ Frag read_frag(const uint8_t* p) {
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
-// ABL: measurement aid of tuning builds (0 in the product): parts of the step left out, results then wrong.
-// 1: operands loaded once per run only, 4: no fp32 / bf16 matrix ops, 8: no fma epilogue, 16: a barrier per step,
-// 64: parts of tiles stored as if whole (no exchange).
-template <int ABL>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_a81w41_fp6_kernel(
     const uint8_t* __restrict__ A6, const uint8_t* __restrict__ W6, int M, int N, int nb, int tiles_m, int tiles_n,
     int panels_m, int panels_n, long long units, float* __restrict__ C, float* __restrict__ partials,
@@ -278,7 +274,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
             pb[i] = W6 + ((size_t)panel_b * nb + k0) * kPanelB;
         }
         auto load_step = [&](int step, Frag (&fa)[2], Frag (&fb)[2]) {
-            const int s = (ABL & 1) ? 0 : min(step, n_steps - 1);  // past the end the last block is read again
+            const int s = min(step, n_steps - 1);  // past the end the last block is read again
 #pragma unroll
             for (int i = 0; i < 2; i++) {
                 fa[i] = read_frag(pa[i] + (size_t)s * kPanelA + lane_a);
@@ -297,7 +293,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         // half 1 blocks 2 and 3 (each half keeps only its own two blocks' pieces), three K slots per block:
         // (s_hi, s_hi, s_lo) against (w_hi, w_lo, w_hi)
         auto min_terms = [&](const uint32_t (&ya)[2][2], const uint32_t (&yb)[2][2]) {
-            if (ABL & 4) return;
             v4i opa[2], opb[2];
 #pragma unroll
             for (int i = 0; i < 2; i++) {
@@ -327,20 +322,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
             const v32f z32 = {0};
 #pragma unroll
             for (int i = 0; i < 2; i++) {
-                v32f Sc = z32;
-                if (!(ABL & 4))
-                    Sc = __builtin_amdgcn_mfma_f32_32x32x1f32(__int_as_float(fa[i][6]), __int_as_float(h ? fb[1][6] : fb[0][6]), z32, 0, 0, 0);
-                else
-                    Sc[0] = __int_as_float(fa[i][6]);
+                const v32f Sc =
+                    __builtin_amdgcn_mfma_f32_32x32x1f32(__int_as_float(fa[i][6]), __int_as_float(h ? fb[1][6] : fb[0][6]), z32, 0, 0, 0);
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
                     const v16f P = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], z16, 2, 2, 0, scale_a, 0, scale_b);
-                    if (ABL & 8) {
-                        acc[i][j][0] += P[0] + Sc[16 * j];
-                    } else {
 #pragma unroll
-                        for (int v = 0; v < 16; v++) acc[i][j][v] = __fmaf_rn(P[v], Sc[16 * j + v], acc[i][j][v]);
-                    }
+                    for (int v = 0; v < 16; v++) acc[i][j][v] = __fmaf_rn(P[v], Sc[16 * j + v], acc[i][j][v]);
                 }
             }
         };
@@ -354,7 +342,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                 for (int u4 = 0; u4 < 4; u4++) {
                     const int step = step0 + u4;
                     if (step >= n_steps) break;  // uniform over the workgroup
-                    if (ABL & 16) __builtin_amdgcn_s_barrier();
                     load_step(step + 1, fa[(u4 + 1) & 1], fb[(u4 + 1) & 1]);
                     const Frag(&ca)[2] = fa[u4 & 1];
                     const Frag(&cb)[2] = fb[u4 & 1];
@@ -389,7 +376,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                 }
         };
 
-        if (n_steps == nb || (ABL & 64)) {
+        if (n_steps == nb) {
             store_tile(acc);
         } else {
             // Part of a tile: park it and count arrivals; the contributor that arrives last adds the parts in
@@ -466,7 +453,7 @@ hipError_t resident_workgroups(int& slots) {
     std::lock_guard<std::mutex> lock(g_mutex);
     if (g_dev[dev].slots == 0) {
         int per_cu = 0, cus = 0;
-        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(&gemm_a81w41_fp6_kernel<0>), kThreads,
+        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(&gemm_a81w41_fp6_kernel), kThreads,
                                                          0);
         if (e != hipSuccess) return e;
         e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
@@ -554,24 +541,9 @@ hipError_t launch_gemm_fp6(const void* a6, const void* w6, float* C, int M, int 
     if (slots > room) slots = (int)room;
     if (slots > ws.max_partials) slots = ws.max_partials;
     const Plan p = make_plan(M, N, K, slots);
-#define A81W41_FP6_LAUNCH(ABL)                                                                                              \
-    hipLaunchKernelGGL(gemm_a81w41_fp6_kernel<ABL>, dim3(p.grid), dim3(kThreads), 0, s, static_cast<const uint8_t*>(a6), \
-                       static_cast<const uint8_t*>(w6), M, N, p.nb, p.tiles_m, p.tiles_n, (M + 31) / 32, (N + 31) / 32, p.units, C, \
-                       ws.partials, ws.arrivals)
-#ifdef A81W41_TUNING
-    switch (tuning_env_int("A81W41_FP6_ABLATE")) {
-#define A81W41_CASE(N)                                                                                                      \
-    case N:                                                                                                                 \
-        A81W41_FP6_LAUNCH(N);                                                                                               \
-        break;
-        A81W41_CASE(1) A81W41_CASE(4) A81W41_CASE(8) A81W41_CASE(12) A81W41_CASE(16) A81W41_CASE(64)
-#undef A81W41_CASE
-        default: A81W41_FP6_LAUNCH(0);
-    }
-#else
-    A81W41_FP6_LAUNCH(0);
-#endif
-#undef A81W41_FP6_LAUNCH
+    hipLaunchKernelGGL(gemm_a81w41_fp6_kernel, dim3(p.grid), dim3(kThreads), 0, s, static_cast<const uint8_t*>(a6),
+                       static_cast<const uint8_t*>(w6), M, N, p.nb, p.tiles_m, p.tiles_n, (M + 31) / 32, (N + 31) / 32, p.units, C,
+                       ws.partials, ws.arrivals);
     return hipGetLastError();
 }
 
