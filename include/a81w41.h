@@ -232,6 +232,40 @@ int a81w41_linear_forward_multi(int n, a81w41_linear *const *layers, const float
  * caller holding Matrix3D<float> buffers uses. */
 int a81w41_linear_forward_host(a81w41_linear *layer, const float *x_host, int M, float *y_host);
 
+/* ---- chains of one-row calls that overlap ----------------------------------
+ * A decode step is a chain of one-row linears, each waiting for the one before
+ * (QwenDecoderLayer.cc:39-105).  Between chain_begin and chain_end the one-row
+ * a81w41_linear_forward / _forward_multi calls of a context's layers are such a
+ * chain: every call still depends on the call before it (its x may be that
+ * call's y), exactly as on a stream, and returns the same bits as outside a
+ * chain, but the launches take turns on two streams, so that a call starts
+ * while its predecessor runs, requests its first weight blocks (which do not
+ * depend on x), and waits for the predecessor inside the kernel.  Measured on
+ * MI355X this hand-over is slower than the kernel boundary it replaces (the
+ * counters and flags of a 256-workgroup launch are served one at a time on the
+ * memory side of the eight L2s), so a chain is an option for experiments, not
+ * the default path of anything.  Rules: calls
+ * name the stream given to chain_begin; M == 1 only; x 16-byte aligned;
+ * buffers the calls read or write are not touched by other work on the GPU
+ * between begin and end; chain_end makes the caller's stream wait for the whole
+ * chain.  Begin ... end may be captured into a HIP graph (stream capture) and
+ * replayed.  Every in-kernel wait is bounded (spin limit in polls of roughly a
+ * microsecond, default 65536): a wait that gives up sets a status word and the
+ * kernels still run to their end; a81w41_context_chain_status synchronises,
+ * reports it (results of that chain are then invalid) and clears it.
+ * No counterpart in the reference, whose calls run one after the other on the
+ * CPU. */
+int a81w41_context_chain_begin(a81w41_context *ctx, void *stream);
+int a81w41_context_chain_end(a81w41_context *ctx);
+int a81w41_context_chain_status(a81w41_context *ctx, int *gave_up);
+int a81w41_context_chain_set_spin_limit(a81w41_context *ctx, unsigned polls);
+/* Test hook for the give-up path: one chained one-row call of `layer` whose wait nothing will
+ * ever satisfy, with a spin limit of `polls`.  The kernel gives up, sets the status word, runs
+ * to its end (y = layer(x) all the same, since x is there) and a81w41_context_chain_status then
+ * reports gave_up = 1.  No chain may be open on the layer's context. */
+int a81w41_context_chain_selfcheck_stuck_wait(a81w41_linear *layer, const float *x_dev, float *y_dev,
+                                              unsigned polls, void *stream);
+
 
 /* ---- the Qwen3 forward pass around the layer ---------------------------------------------
  * Replaces Qwen3ForCausalLM / Qwen3Model / Qwen3DecoderLayer / Qwen3Attention
@@ -280,15 +314,21 @@ int a81w41_qwen3_set_norm(a81w41_qwen3 *model, int layer, int which, const float
 int a81w41_qwen3_set_embedding(a81w41_qwen3 *model, const uint16_t *table_fp16);
 /* Test switches: each keeps one fusion of the one-token / prefill pass off, so that the fused
  * pass can be compared with the separate kernels, or fixes the attention's key split.  The
- * results of a pass do not change by a bit with UNFUSED, ATTN_FP32 and NO_PAIR. */
+ * results of a pass do not change by a bit with UNFUSED, ATTN_FP32, NO_PAIR and CHAIN.
+ * With CHAIN on, the one-token pass runs its linears and attention as a chain of overlapping
+ * launches (see a81w41_context_chain_begin); a81w41_qwen3_chain_status reports whether a wait
+ * of such a chain has given up since the last call. */
 enum {
     A81W41_QWEN3_OPT_UNFUSED = 0,          /* separate elementwise kernels and quantiser launches */
     A81W41_QWEN3_OPT_ATTN_FP32 = 1,        /* one-token attention writes fp32, o_proj quantises it */
     A81W41_QWEN3_OPT_NO_PAIR = 2,          /* gate_up writes fp32, down_proj's prologue does SiLU*mul */
     A81W41_QWEN3_OPT_VECTOR_ATTENTION = 3, /* prefill attention on the vector kernel */
-    A81W41_QWEN3_OPT_ATTENTION_SPLIT = 4   /* value 1..16: shares per head of the one-token attention; 0: automatic */
+    A81W41_QWEN3_OPT_ATTENTION_SPLIT = 4,  /* value 1..16: shares per head of the one-token attention; 0: automatic */
+    A81W41_QWEN3_OPT_CHAIN = 5,            /* one-token pass as a chain of overlapping launches (off by default: slower) */
+    A81W41_QWEN3_OPT_CHAIN_SPIN_LIMIT = 6  /* value: polls before an in-kernel wait of the chained pass gives up; 0: default */
 };
 int a81w41_qwen3_set_option(a81w41_qwen3 *model, int option, int value);
+int a81w41_qwen3_chain_status(a81w41_qwen3 *model, int *gave_up); /* synchronises */
 /* Parity hook: copies the first `count` floats of one of the model's activation buffers to the host
  * after the work enqueued so far has finished.  After a pass the buffers hold what the LAST layer left
  * (the fused passes skip some of them: switch A81W41_QWEN3_OPT_UNFUSED on to have every stage written):

@@ -53,6 +53,11 @@ SIGNATURES = {
     "a81w41_linear_set_kernel": (_i, [_vp, _i]),
     "a81w41_linear_forward_multi": (_i, [_i, C.POINTER(_vp), _vp, _i, C.POINTER(_vp), _vp]),
     "a81w41_linear_forward_host": (_i, [_vp, _vp, _i, _vp]),
+    "a81w41_context_chain_begin": (_i, [_vp, _vp]),
+    "a81w41_context_chain_end": (_i, [_vp]),
+    "a81w41_context_chain_status": (_i, [_vp, C.POINTER(_i)]),
+    "a81w41_context_chain_set_spin_limit": (_i, [_vp, C.c_uint]),
+    "a81w41_context_chain_selfcheck_stuck_wait": (_i, [_vp, _vp, _vp, C.c_uint, _vp]),
     "a81w41_qwen3_create": (_i, [_vp, C.POINTER(_vp)]),
     "a81w41_qwen3_load": (_i, [C.c_char_p, _vp, C.POINTER(_vp)]),
     "a81w41_qwen3_destroy": (None, [_vp]),
@@ -61,6 +66,7 @@ SIGNATURES = {
     "a81w41_qwen3_set_norm": (_i, [_vp, _i, _i, _vp]),
     "a81w41_qwen3_set_embedding": (_i, [_vp, _vp]),
     "a81w41_qwen3_set_option": (_i, [_vp, _i, _i]),
+    "a81w41_qwen3_chain_status": (_i, [_vp, C.POINTER(_i)]),
     "a81w41_qwen3_read_buffer": (_i, [_vp, _i, _vp, _sz]),
     "a81w41_qwen3_reset": (_i, [_vp]),
     "a81w41_qwen3_forward": (_i, [_vp, _vp, _i, _vp]),

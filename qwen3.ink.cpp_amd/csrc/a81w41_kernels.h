@@ -5,6 +5,8 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include "chain.h"
+
 namespace a81w41 {
 
 // Environment overrides of the kernel selection exist in tuning builds only (make TUNING=1); the
@@ -64,6 +66,45 @@ hipError_t launch_gemv_add_norm(const float* x, const GemvPrologue& pro, void* a
 bool gemv_pair_fits(int N, int K);
 hipError_t launch_gemv_add_norm_silu_pair(const float* x, const GemvPrologue& pro, const void* B_gate_up, int N, int K,
                                           hipStream_t s);
+int gemv_waves_per_group_log2(int nb_n, int nb_k, bool paired_output);
+
+// ---- chains of overlapping launches, host side (chain.hip; the device side is in chain.h) ----------------------
+// Between chain_begin and chain_end every launch is a link: it goes to the stream chain_next names (the caller's
+// stream and the chain's own side stream in turn), waits inside the kernel for the link before it, and its
+// workgroup count is reported with chain_launched.  Works under stream capture (the side stream joins the capture
+// through the fork event and leaves it through the join event).
+constexpr int kChainRing = 4;  // completion counters in rotation; the status word follows them
+struct ChainState {
+    unsigned* counters = nullptr;  // device
+    hipStream_t side = nullptr, main = nullptr;
+    hipEvent_t fork = nullptr, join = nullptr;
+    bool open = false;
+    int n = 0;               // launches of the open chain so far
+    unsigned prev_grid = 0;  // workgroups of the last one
+    unsigned spin_limit = 1u << 16;  // polls (about a microsecond each) before a wait gives up
+    int cus = 0;
+};
+hipError_t chain_create(ChainState* st);
+void chain_destroy(ChainState* st);
+hipError_t chain_begin(ChainState* st, hipStream_t main);
+ChainLink chain_next(const ChainState* st, hipStream_t* stream);
+void chain_launched(ChainState* st, unsigned grid);
+hipError_t chain_end(ChainState* st);  // the caller's stream waits for the side stream; clears the last counter
+// Synchronises both streams; *gave_up = some wait of a chain since the last call gave up (counters are then reset).
+hipError_t chain_status(ChainState* st, bool* gave_up);
+// The same launches as links of a chain of overlapping launches (chain.h, gemv_chain_a81w41.hip): same bits as
+// the plain launches while K < 16384; at most `cus` workgroups of 8 waves; *grid_out = workgroups launched (what
+// the next link waits for).  gemv_chain_fits: K a multiple of 64, the quantised row within 64 KiB of LDS, and
+// for the add + norm prologue K <= 4096.
+bool gemv_chain_fits(int K, bool add_norm);
+hipError_t launch_gemv_chain_blob(const void* A, const void* B, float* C, int N, int K, const ChainLink& link, int cus,
+                                  unsigned* grid_out, hipStream_t s);
+hipError_t launch_gemv_chain_fused(const float* x, void* a_out, int n_mat, const void* const* Bs, float* const* Cs,
+                                   const int* Ns, int K, const ChainLink& link, int cus, unsigned* grid_out, hipStream_t s);
+hipError_t launch_gemv_chain_add_norm(const float* x, const GemvPrologue& pro, void* a_out, const void* B, float* C, int N,
+                                      int K, const ChainLink& link, int cus, unsigned* grid_out, hipStream_t s);
+hipError_t launch_gemv_chain_add_norm_silu_pair(const float* x, const GemvPrologue& pro, const void* B_gate_up, int N, int K,
+                                                const ChainLink& link, int cus, unsigned* grid_out, hipStream_t s);
 // Scratch of the GEMM's K-split path: partial tiles and their arrival counters (zero between launches).
 // Launches that share a scratch must not overlap in time.
 struct GemmScratch {
@@ -133,6 +174,7 @@ struct a81w41_context;
 namespace a81w41 {
 // The K-split scratch a context owns, and its A6 scratch (capi.cpp).
 const GemmScratch& context_gemm_scratch(const a81w41_context* ctx);
+ChainState* context_chain(a81w41_context* ctx);
 void* context_a6_scratch(const a81w41_context* ctx);
 }  // namespace a81w41
 struct a81w41_linear;
@@ -176,7 +218,8 @@ hipError_t launch_attention_prefill(const float* q, int q_row_stride, const void
 // the fp16-parameter quantiser would make of it (out is then not written).
 hipError_t launch_attention_one_token(const float* qkv, int n_q, int n_kv, const float* q_w, const float* k_w,
                                       const float* cos_t, const float* sin_t, const int* pos_dev, void* k_cache, void* v_cache,
-                                      float* out, void* q_out, int max_seq, float eps, float scale, hipStream_t s);
+                                      float* out, void* q_out, int max_seq, float eps, float scale, hipStream_t s,
+                                      const ChainLink* link = nullptr);  // link: the launch is a link of a chain (chain.h)
 // The same with the context of every head cut into `splits` (<= kAttentionMaxSplits) shares, one workgroup
 // each, for long contexts.  partials: n_q * splits * 132 floats; arrivals: n_q counters, zero before the
 // first launch (every launch leaves them zero).  Launches that share them must not overlap in time.
@@ -184,7 +227,8 @@ constexpr int kAttentionMaxSplits = 16;
 hipError_t launch_attention_one_token_split(const float* qkv, int n_q, int n_kv, const float* q_w, const float* k_w,
                                             const float* cos_t, const float* sin_t, const int* pos_dev, void* k_cache,
                                             void* v_cache, float* out, void* q_out, float* partials, unsigned* arrivals,
-                                            int splits, int max_seq, float eps, float scale, hipStream_t s);
+                                            int splits, int max_seq, float eps, float scale, hipStream_t s,
+                                            const ChainLink* link = nullptr);
 hipError_t launch_silu_mul(const float* gate_up, float* out, int M, int inter, hipStream_t s);
 // silu(gate) * up as 80 B activation blocks of the [M][inter] result.  inter % 64 == 0, gate_up 16-byte aligned.
 hipError_t launch_silu_mul_quant(const float* gate_up, void* q_out, int M, int inter, hipStream_t s);

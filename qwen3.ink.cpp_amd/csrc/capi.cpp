@@ -138,6 +138,8 @@ struct a81w41_context {
     float* x_stage = nullptr;  // device staging for forward_host
     float* y_stage = nullptr;
     size_t x_bytes = 0, y_bytes = 0;
+    a81w41::ChainState chain;  // overlapping dependent launches (a81w41_context_chain_*), created at first use
+    bool chain_ready = false;
 };
 
 struct a81w41_linear {
@@ -152,6 +154,13 @@ struct a81w41_linear {
 namespace a81w41 {
 const GemmScratch& context_gemm_scratch(const a81w41_context* ctx) { return ctx->gemm_scratch; }
 void* context_a6_scratch(const a81w41_context* ctx) { return ctx->a6_scratch; }
+ChainState* context_chain(a81w41_context* ctx) {
+    if (!ctx->chain_ready) {
+        if (chain_create(&ctx->chain) != hipSuccess) return nullptr;
+        ctx->chain_ready = true;
+    }
+    return &ctx->chain;
+}
 const void* linear_w6(const a81w41_linear* layer) { return layer->w6; }
 bool linear_block_scaled(const a81w41_linear* l, int M) {
     if (!l->w6 || M < kGemmFp6MinRows || l->kernel_choice == A81W41_KERNEL_INT8) return false;
@@ -437,6 +446,11 @@ int a81w41_context_create(int max_rows, int max_cols, a81w41_context** out) {
         (void)hipFree(ctx->act_scratch);
         return hip_fail(e, "hipMalloc(activation scratch)");
     }
+    // the chain's stream, events and counters exist from the start, so that a chain can be opened under stream capture
+    if (!a81w41::context_chain(ctx.get())) {
+        a81w41_context_destroy(ctx.release());
+        return fail(A81W41_ERR_HIP, "cannot create the chain's stream, events and counters");
+    }
     *out = ctx.release();
     return A81W41_OK;
 }
@@ -444,6 +458,7 @@ int a81w41_context_create(int max_rows, int max_cols, a81w41_context** out) {
 void a81w41_context_destroy(a81w41_context* ctx) {
     if (!ctx) return;
     a81w41::gemm_scratch_destroy(&ctx->gemm_scratch);
+    if (ctx->chain_ready) a81w41::chain_destroy(&ctx->chain);
     (void)hipFree(ctx->act_scratch);
     (void)hipFree(ctx->a6_scratch);
     (void)hipFree(ctx->x_stage);
@@ -539,6 +554,86 @@ int a81w41_linear_out_features(const a81w41_linear* l) { return l ? l->N : 0; }
 const void* a81w41_linear_weight_fp16_dev(const a81w41_linear* l) { return l ? l->w16 : nullptr; }
 const void* a81w41_linear_weight_fp32_dev(const a81w41_linear* l) { return l ? l->w32 : nullptr; }
 
+// One-row call on a context whose chain is open: the fused quantise + contract launch as the chain's next link.
+static int chained_forward(a81w41_context* ctx, int n, const void* const* Bs, float* const* Cs, const int* Ns, int K,
+                           const float* x_dev, int M, void* stream) {
+    a81w41::ChainState& ch = ctx->chain;
+    if (M != 1) return fail(A81W41_ERR_INVALID_ARG, "a chain is open on this context: only one-row calls (M = 1), got M = %d", M);
+    if (static_cast<hipStream_t>(stream) != ch.main)
+        return fail(A81W41_ERR_INVALID_ARG, "a chain is open on this context: calls must name the stream it was opened on");
+    for (int j = 0; j < n; j++) {
+        if (!Bs[j]) return fail(A81W41_ERR_INVALID_ARG, "layer has no fp16-parameter blob (needed for M == 1)");
+        if (reinterpret_cast<uintptr_t>(Cs[j]) & 3) return fail(A81W41_ERR_INVALID_ARG, "y must be 4-byte aligned");
+    }
+    if ((reinterpret_cast<uintptr_t>(x_dev) & 15) || !a81w41::gemv_chain_fits(K, false))
+        return fail(A81W41_ERR_INVALID_ARG, "a chained call needs x 16-byte aligned and K <= 40960, got K = %d", K);
+    if (int st = check_device()) return st;
+    hipStream_t s = nullptr;
+    const a81w41::ChainLink link = a81w41::chain_next(&ch, &s);
+    unsigned grid = 0;
+    HIP_TRY(a81w41::launch_gemv_chain_fused(x_dev, ctx->act_scratch, n, Bs, Cs, Ns, K, link, ch.cus, &grid, s));
+    a81w41::chain_launched(&ch, grid);
+    return A81W41_OK;
+}
+
+int a81w41_context_chain_begin(a81w41_context* ctx, void* stream) {
+    if (!ctx) return fail(A81W41_ERR_INVALID_ARG, "null context");
+    if (int st = check_device()) return st;
+    a81w41::ChainState* ch = a81w41::context_chain(ctx);
+    if (!ch) return fail(A81W41_ERR_HIP, "cannot create the chain's stream, events and counters");
+    if (ch->open) return fail(A81W41_ERR_INVALID_ARG, "a chain is already open on this context");
+    HIP_TRY(a81w41::chain_begin(ch, static_cast<hipStream_t>(stream)));
+    return A81W41_OK;
+}
+
+int a81w41_context_chain_end(a81w41_context* ctx) {
+    if (!ctx || !ctx->chain_ready || !ctx->chain.open) return fail(A81W41_ERR_INVALID_ARG, "no chain is open on this context");
+    HIP_TRY(a81w41::chain_end(&ctx->chain));
+    return A81W41_OK;
+}
+
+int a81w41_context_chain_status(a81w41_context* ctx, int* gave_up) {
+    if (!ctx || !gave_up) return fail(A81W41_ERR_INVALID_ARG, "null argument");
+    *gave_up = 0;
+    if (!ctx->chain_ready) return A81W41_OK;
+    if (ctx->chain.open) return fail(A81W41_ERR_INVALID_ARG, "close the chain first");
+    bool bad = false;
+    HIP_TRY(a81w41::chain_status(&ctx->chain, &bad));
+    *gave_up = bad ? 1 : 0;
+    return A81W41_OK;
+}
+
+int a81w41_context_chain_selfcheck_stuck_wait(a81w41_linear* l, const float* x_dev, float* y_dev, unsigned polls, void* stream) {
+    if (!l || !x_dev || !y_dev) return fail(A81W41_ERR_INVALID_ARG, "null pointer");
+    a81w41_context* ctx = l->ctx;
+    a81w41::ChainState* ch = a81w41::context_chain(ctx);
+    if (!ch) return fail(A81W41_ERR_HIP, "cannot create the chain's stream, events and counters");
+    if (ch->open) return fail(A81W41_ERR_INVALID_ARG, "close the chain first");
+    if (!l->w16 || (reinterpret_cast<uintptr_t>(x_dev) & 15) || (reinterpret_cast<uintptr_t>(y_dev) & 3) ||
+        !a81w41::gemv_chain_fits(l->K, false))
+        return fail(A81W41_ERR_INVALID_ARG, "needs the fp16-parameter blob, x 16-byte aligned, K <= 40960");
+    if (int st = check_device()) return st;
+    a81w41::ChainLink link;
+    link.wait = ch->counters;  // zero at rest, and nothing will count on it
+    link.wait_for = 1;
+    link.status = ch->counters + a81w41::kChainRing;
+    link.spin_limit = polls;
+    const void* Bs[1] = {l->w16};
+    float* Cs[1] = {y_dev};
+    HIP_TRY(a81w41::launch_gemv_chain_fused(x_dev, ctx->act_scratch, 1, Bs, Cs, &l->N, l->K, link, ch->cus, nullptr,
+                                            static_cast<hipStream_t>(stream)));
+    return A81W41_OK;
+}
+
+int a81w41_context_chain_set_spin_limit(a81w41_context* ctx, unsigned polls) {
+    if (!ctx) return fail(A81W41_ERR_INVALID_ARG, "null context");
+    a81w41::ChainState* ch = a81w41::context_chain(ctx);
+    if (!ch) return fail(A81W41_ERR_HIP, "cannot create the chain's stream, events and counters");
+    if (ch->open) return fail(A81W41_ERR_INVALID_ARG, "close the chain first");
+    ch->spin_limit = polls;
+    return A81W41_OK;
+}
+
 int a81w41_linear_forward(a81w41_linear* l, const float* x_dev, int M, float* y_dev, void* stream) {
     if (!l || !x_dev || !y_dev) return fail(A81W41_ERR_INVALID_ARG, "null pointer");
     if (M < 1) return fail(A81W41_ERR_INVALID_ARG, "M must be >= 1, got %d", M);
@@ -546,6 +641,11 @@ int a81w41_linear_forward(a81w41_linear* l, const float* x_dev, int M, float* y_
     if ((int64_t)M * l->K > ctx->max_elems)
         return fail(A81W41_ERR_INVALID_ARG, "M*K = %lld exceeds the context's activation scratch (%lld)",
                     (long long)M * l->K, (long long)ctx->max_elems);
+    if (ctx->chain_ready && ctx->chain.open) {  // a link of the context's open chain
+        const void* Bs[1] = {l->w16};
+        float* Cs[1] = {y_dev};
+        return chained_forward(ctx, 1, Bs, Cs, &l->N, l->K, x_dev, M, stream);
+    }
     // QwenOperator.cc:96-120: the precision of the activation parameters follows M.
     if (M > 1) {
         if (!l->w32) return fail(A81W41_ERR_INVALID_ARG, "layer has no fp32-parameter blob (needed for M > 1)");
@@ -598,6 +698,19 @@ int a81w41_linear_forward_multi(int n, a81w41_linear* const* layers, const float
             return fail(A81W41_ERR_INVALID_ARG, "layers of one call must share K and the context");
     }
     a81w41_linear* l0 = layers[0];
+    if (l0->ctx->chain_ready && l0->ctx->chain.open) {
+        if (n > a81w41::kGemvMaxBatch)
+            return fail(A81W41_ERR_INVALID_ARG, "at most %d layers per call while a chain is open", a81w41::kGemvMaxBatch);
+        const void* Bs[a81w41::kGemvMaxBatch];
+        float* Cs[a81w41::kGemvMaxBatch];
+        int Ns[a81w41::kGemvMaxBatch];
+        for (int j = 0; j < n; j++) {
+            Bs[j] = layers[j]->w16;
+            Cs[j] = ys_dev[j];
+            Ns[j] = layers[j]->N;
+        }
+        return chained_forward(l0->ctx, n, Bs, Cs, Ns, l0->K, x_dev, M, stream);
+    }
     const bool one_launch = M == 1 && (reinterpret_cast<uintptr_t>(x_dev) & 15) == 0 &&
                             a81w41::gemv_lds_bytes(l0->K) <= a81w41::kLdsLimitBytes;
     if (!one_launch) {  // same results, one call per layer (each re-quantises x into the scratch)

@@ -39,8 +39,7 @@
 // kernel: same blocks, codes read as code - 8, no min term.  The lane subtracts eight
 // times the sum of the activation bytes it dotted, which keeps the block dots exact,
 // and never touches the min / scaled-sum fields (that variant's writers leave them unset).
-#include "a81w41_kernels.h"
-#include "quantize_common.h"
+#include "gemv_common.h"
 
 #include <cstdio>
 #include <cstdlib>
@@ -48,88 +47,7 @@
 namespace a81w41 {
 namespace {
 
-constexpr int kMaxWaves = 16;
-constexpr int kBlocksPerStep = 16;  // blocks a wave consumes per step
-// LDS image of one activation super-block: for pp = 0,1: 4 q_low words (packs
-// pp,pp+2,pp+4,pp+6), 4 q_high words, dA_pp, sA_pp, 2 pad words  -> 2 x 48 B.
-constexpr int kLdsWordsPerSb = 24;
-
-__device__ __forceinline__ int dpp_xor2(int v) { return dpp_i<kDppXor2>(v); }
-
-struct BlockLoads {
-    uint4 w[4];    // packs pp, pp+2, pp+4, pp+6 (this lane's 4 columns)
-    uint2 sc, mn;  // 4 fp16 scales / mins of 32-block lh = pp, columns 4h..4h+3
-};
-
-template <bool MINS>
-__device__ __forceinline__ void load_block(BlockLoads& L, const uint8_t* blk, int sub, bool valid) {
-    if (valid) {
-        const int h = sub & 1, pp = sub >> 1;
-        const uint8_t* q = blk + 64 + 16 * h + 32 * pp;
-#pragma unroll
-        for (int j = 0; j < 4; j++) L.w[j] = *reinterpret_cast<const uint4*>(q + 64 * j);
-        L.sc = *reinterpret_cast<const uint2*>(blk + 8 * sub);
-        L.mn = MINS ? *reinterpret_cast<const uint2*>(blk + 32 + 8 * sub) : make_uint2(0, 0);
-    } else {
-#pragma unroll
-        for (int j = 0; j < 4; j++) L.w[j] = make_uint4(0, 0, 0, 0);
-        L.sc = make_uint2(0, 0);
-        L.mn = make_uint2(0, 0);
-    }
-}
-
-// Up to kGemvMaxBatch weight matrices that share the activation row (and K) are
-// contracted by one launch: their column groups are numbered back to back.
-struct GemvBatch {
-    const uint8_t* B[kGemvMaxBatch];
-    float* C[kGemvMaxBatch];
-    int end[kGemvMaxBatch];  // exclusive end of matrix j's column groups in the joint numbering
-};
-
-struct GroupRef {
-    const uint8_t* B;  // first block of the column group
-    float* C;          // its 8 outputs
-};
-
-__device__ __forceinline__ GroupRef locate(const GemvBatch& bt, int g, int nb_k) {
-    int j = 0, first = 0;
-#pragma unroll
-    for (int t = 0; t + 1 < kGemvMaxBatch; t++) {
-        if (g >= bt.end[t]) {
-            j = t + 1;
-            first = bt.end[t];
-        }
-    }
-    const int lg = g - first;
-    return {bt.B[j] + (size_t)lg * nb_k * kWBlock16, bt.C[j] + (size_t)lg * 8};
-}
-
-// Workgroup barrier that orders LDS traffic only: every LDS access this wave has issued is done, global
-// loads stay in flight.  __syncthreads() would drain them too (loads and stores share one counter),
-// i.e. wait for the weight blocks requested ahead at every barrier.
-__device__ __forceinline__ void lds_barrier() {
-    __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt = 0; vector-memory and export counters left alone
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-}
-
-// LDS word of q word (32-block lh, pack p) inside a super-block image.
-__device__ __forceinline__ int lds_q_word(int lh, int p) { return 12 * (p & 1) + 4 * lh + (p >> 1); }
-
-// What the activation row is made from (template parameter PRO of the kernel).
-// kProBlobA80: a 72 B-block blob again, contracted the A80W40 way.
-// kProAddNormPair: kProAddNorm in front, paired gate|up output behind.
-enum : int { kProBlob = 0, kProX = 1, kProSiluMul = 2, kProAddNorm = 3, kProBlobA80 = 4, kProAddNormPair = 5 };
-
-// Paired output: the groups a workgroup walks, in its own order v = b*slots + slot + i*g_stride
-// (grid = N/64 workgroups, 8/slots iterations each): workgroup b's w-th group (w = i*slots + slot) is
-// gate group 4b + w for w < 4, up group 4b + w - 4 after that.
-__device__ __forceinline__ int pair_group(int v, int g_stride, int slots, int nb_n) {
-    const int i = v / g_stride, rem = v - i * g_stride;
-    const int b = rem / slots, w = i * slots + (rem - b * slots);
-    return w < 4 ? 4 * b + w : (nb_n >> 1) + 4 * b + (w - 4);
-}
+using namespace gemv;
 
 // Argument order: the leading pointer and integers are handed over in scalar registers at dispatch
 // (kernel-argument preloading, switched on in the Makefile; it stops at the first struct), so the row
@@ -225,28 +143,33 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_a81w41_fp16_kernel(const voi
             if (kAddNorm) {  // the whole row is in this one chunk (the launcher checks)
                 const bool has_res = pro.res_in != nullptr;
                 float4* o4 = reinterpret_cast<float4*>(pro.res_out);
-                float ss = 0.f;
+                // sum of squares in an order that does not depend on the workgroup's width: per float4, then over
+                // each aligned group of 64 float4 (a wave's slice), then over the groups by the same tree
+                float ss[kChunk];
 #pragma unroll
                 for (int u = 0; u < kChunk; u++) {
                     const int i = base + u * kThreads + tid;
+                    ss[u] = 0.f;
                     if (i < n_vec) {
                         if (has_res) {
                             const float4 r = rr[kAddNorm ? u : 0];
                             v[u].x += r.x; v[u].y += r.y; v[u].z += r.z; v[u].w += r.w;
                         }
                         if (blockIdx.x == 0) o4[i] = v[u];
-                        ss += v[u].x * v[u].x + v[u].y * v[u].y + v[u].z * v[u].z + v[u].w * v[u].w;
+                        ss[u] = v[u].x * v[u].x + v[u].y * v[u].y + v[u].z * v[u].z + v[u].w * v[u].w;
                     }
                 }
-#pragma unroll
-                for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
                 float* part = reinterpret_cast<float*>(lds + nb_k * kLdsWordsPerSb);  // the reduction area, idle now
-                if (lane == 0) part[wave] = ss;
-                lds_barrier();
-                float total = 0.f;
 #pragma unroll
-                for (int w = 0; w < kWaves; w++) total += part[w];
+                for (int u = 0; u < kChunk; u++) {
+                    if (base + u * kThreads >= n_vec) break;  // empty slice (uniform over the workgroup)
+                    ss[u] = wave_sum_fixed_order(ss[u]);
+                    if (lane == 0) part[u * kWaves + wave] = ss[u];
+                }
                 lds_barrier();
+                sum_groups_fixed_order(part, (n_vec + 63) / 64, wave, lane);
+                lds_barrier();
+                const float total = part[64];
                 const float inv = 1.0f / sqrtf(total / (float)(64 * nb_k) + pro.eps);
 #pragma unroll
                 for (int u = 0; u < kChunk; u++) {
@@ -339,64 +262,11 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_a81w41_fp16_kernel(const voi
             load_block<!kA80>(nxt, locate(bt, png, nb_k).B + (size_t)nblk * kWBlock16, sub, ng < nb_n && nblk < nb_k);
         }
 
-        const uint32_t* a = lds + (valid ? blk : 0) * kLdsWordsPerSb + 12 * pp;
-        const uint4 aql = *reinterpret_cast<const uint4*>(a);
-        const uint4 aqh = *reinterpret_cast<const uint4*>(a + 4);
-        const float2 par = *reinterpret_cast<const float2*>(a + 8);  // dA_pp, sA_pp
-        const uint32_t al[4] = {aql.x, aql.y, aql.z, aql.w};
-        const uint32_t ah[4] = {aqh.x, aqh.y, aqh.z, aqh.w};
-
-        int il[4] = {0, 0, 0, 0}, ih[4] = {0, 0, 0, 0};
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const uint32_t w4[4] = {cur.w[j].x, cur.w[j].y, cur.w[j].z, cur.w[j].w};
-#pragma unroll
-            for (int c = 0; c < 4; c++) {
-                const uint32_t lo = w4[c] & 0x0f0f0f0fu;
-                const uint32_t hi = (w4[c] >> 4) & 0x0f0f0f0fu;
-                il[c] = __builtin_amdgcn_sdot4((int)lo, (int)al[j], il[c], false);
-                ih[c] = __builtin_amdgcn_sdot4((int)hi, (int)ah[j], ih[c], false);
-            }
-        }
-        if (kA80) {  // sum((code - 8) q) = sum(code q) - 8 sum(q), over the bytes this lane dotted
-            int sl = 0, sh = 0;
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                sl = __builtin_amdgcn_sdot4(0x01010101, (int)al[j], sl, false);
-                sh = __builtin_amdgcn_sdot4(0x01010101, (int)ah[j], sh, false);
-            }
-#pragma unroll
-            for (int c = 0; c < 4; c++) {
-                il[c] -= 8 * sl;
-                ih[c] -= 8 * sh;
-            }
-        }
-        const uint32_t sc[2] = {cur.sc.x, cur.sc.y}, mn[2] = {cur.mn.x, cur.mn.y};
-#pragma unroll
-        for (int c = 0; c < 4; c++) {
-            il[c] += dpp_xor2(il[c]);  // exact int32 block dots of columns 4h+c
-            ih[c] += dpp_xor2(ih[c]);
-            const int idot = pp ? ih[c] : il[c];
-            const float dW = f16_bits_to_f32((sc[c >> 1] >> (16 * (c & 1))) & 0xffff);
-            const float mW = f16_bits_to_f32((mn[c >> 1] >> (16 * (c & 1))) & 0xffff);
-            const float s = __fmul_rn(par.x, dW);
-            acc[c] = __fmaf_rn((float)idot, s, acc[c]);
-            if (!kA80) acc[c] = __fmaf_rn(mW, par.y, acc[c]);
-        }
+        consume_block<kA80>(cur, lds + (valid ? blk : 0) * kLdsWordsPerSb + 12 * pp, pp, acc);
         cur = nxt;
 
         if (nsi == 0) {  // group finished (uniform over the workgroup)
-            // Sum inside each row of 16 lanes over the lanes that share h: rotate by 8 and 4
-            // (keeps lane % 4), then swap the two pp lanes.  Every lane of a row ends up with
-            // the row's total for its h; lanes 0 and 1 of each row publish it.
-#pragma unroll
-            for (int c = 0; c < 4; c++) {
-                float v = acc[c];
-                v += dpp_f<0x128>(v);  // row_ror:8
-                v += dpp_f<0x124>(v);  // row_ror:4
-                v += dpp_f<kDppXor2>(v);
-                acc[c] = v;
-            }
+            sum_rows_of_16(acc);
             float* r = red + parity * (kWaves * 32);
             if ((lane & 15) < 2) {
                 float4* dst = reinterpret_cast<float4*>(r + wave * 32 + (lane >> 4) * 8 + 4 * (lane & 1));
@@ -471,6 +341,25 @@ GemvTune pick_tune(int nb_n, int nb_k) {
     return {16, 256, 0};
 }
 
+}  // namespace
+
+// Waves per column group of a launch over nb_n groups of nb_k blocks: a power of two, at most the workgroup
+// width and the number of 16-block steps.  It fixes the order in which a column's partial sums are added.
+int gemv_waves_per_group_log2(int nb_n, int nb_k, bool paired_output) {
+    const GemvTune t = pick_tune(nb_n, nb_k);
+    const int n_steps = (nb_k + kBlocksPerStep - 1) / kBlocksPerStep;
+    int wpg_log2 = 0;
+    const int want = t.wpg > 0 ? t.wpg : n_steps;
+    while ((2 << wpg_log2) <= want && (2 << wpg_log2) <= t.waves) wpg_log2++;
+    // paired output: a workgroup walks its eight groups in 8 / slots rounds, so at most eight groups at a time
+    // (short rows in wide workgroups -- hidden 1024 with 16 waves -- would otherwise have sixteen)
+    if (paired_output)
+        while ((t.waves >> wpg_log2) > 8) wpg_log2++;
+    return wpg_log2;
+}
+
+namespace {
+
 template <int PRO>
 hipError_t launch(const void* a_or_x, void* a_out, int n_mat, const void* const* Bs, float* const* Cs,
                   const int* Ns, int K, const GemvPrologue& pro, hipStream_t s) {
@@ -487,15 +376,7 @@ hipError_t launch(const void* a_or_x, void* a_out, int n_mat, const void* const*
     const GemvTune t = pick_tune(nb_n, nb_k);
     // the add + norm prologue holds the whole row in one chunk of 4 float4 per thread
     if ((PRO == kProAddNorm || PRO == kProAddNormPair) && 16 * nb_k > 4 * 64 * t.waves) return hipErrorInvalidValue;
-    // waves per group: a power of two, at most the workgroup width and the number of 16-block steps
-    const int n_steps = (nb_k + kBlocksPerStep - 1) / kBlocksPerStep;
-    int wpg_log2 = 0;
-    const int want = t.wpg > 0 ? t.wpg : n_steps;
-    while ((2 << wpg_log2) <= want && (2 << wpg_log2) <= t.waves) wpg_log2++;
-    // paired output: a workgroup walks its eight groups in 8 / slots rounds, so at most eight groups at a time
-    // (short rows in wide workgroups -- hidden 1024 with 16 waves -- would otherwise have sixteen)
-    if (PRO == kProAddNormPair)
-        while ((t.waves >> wpg_log2) > 8) wpg_log2++;
+    const int wpg_log2 = gemv_waves_per_group_log2(nb_n, nb_k, PRO == kProAddNormPair);
     const int slots = t.waves >> wpg_log2;
     const int wgs = (nb_n + slots - 1) / slots;
     int grid = wgs < t.max_grid ? wgs : t.max_grid;

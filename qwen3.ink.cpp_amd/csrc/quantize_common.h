@@ -80,7 +80,9 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t bits16) {
 
 // One value per lane, 32 consecutive lanes (an aligned half wave, all active) holding one 32-block of
 // a row: the fp16-parameter quantiser (quantize_row_q8_1_repack_fp16, quantized_gemx_kernels.cc:693-801)
-// written into the row's 72 B blocks.  col = the value's index in the row.
+// written into the row's 72 B blocks.  col = the value's index in the row.  AGENT: the stores are agent-scope
+// stores (a consumer on another XCD reads the blocks while this kernel is still running).
+template <bool AGENT = false>
 __device__ __forceinline__ void store_quantized_value_fp16(uint8_t* __restrict__ blob, int col, float v) {
     float amax = fabsf(v);
 #pragma unroll
@@ -93,13 +95,21 @@ __device__ __forceinline__ void store_quantized_value_fp16(uint8_t* __restrict__
     for (int off = 16; off > 0; off >>= 1) sum += (unsigned)__shfl_xor((int)sum, off, 64);
     uint8_t* blk = blob + (col >> 6) * 72;
     const int h = (col >> 5) & 1, i = col & 31;
-    blk[8 + 32 * h + i] = (uint8_t)sat8(r);
+    if (AGENT)
+        __hip_atomic_store(blk + 8 + 32 * h + i, (uint8_t)sat8(r), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else
+        blk[8 + 32 * h + i] = (uint8_t)sat8(r);
     if (i == 0) {
         float ssum = __fmul_rn(d, (float)(int)sum);
         asm volatile("" : "+v"(ssum));  // keep the fp32 product: two roundings, as in the reference
         uint16_t* par = reinterpret_cast<uint16_t*>(blk);
-        par[h] = f32_to_f16_bits(d);
-        par[2 + h] = f32_to_f16_bits(ssum);
+        if (AGENT) {
+            __hip_atomic_store(par + h, f32_to_f16_bits(d), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(par + 2 + h, f32_to_f16_bits(ssum), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+            par[h] = f32_to_f16_bits(d);
+            par[2 + h] = f32_to_f16_bits(ssum);
+        }
     }
 }
 

@@ -69,7 +69,8 @@ struct a81w41_qwen3 {
     int cu_count = 0;  // of the device the model lives on
     // Switches of a81w41_qwen3_set_option: each keeps a fusion off (or fixes the attention's key split) so
     // that tests can compare the fused pass with the separate kernels bit for bit.
-    bool opt_unfused = false, opt_attn_fp32 = false, opt_no_pair = false, opt_vector_attention = false;
+    bool opt_unfused = false, opt_attn_fp32 = false, opt_no_pair = false, opt_vector_attention = false, opt_chain = false;
+    unsigned opt_spin_limit = 0;  // 0: the chain's default
     int opt_attention_split = 0;
     int qkv_dim() const { return (cfg.n_q_heads + 2 * cfg.n_kv_heads) * kHeadDim; }
 };
@@ -188,15 +189,16 @@ int enqueue_pass(a81w41_qwen3* m, int M, hipStream_t s) {
 // the new residual while the other workgroups still read the old one.
 // q/k norm + rotation + cache append + attention for the one new token, in one workgroup per head or,
 // for long contexts, in `splits` workgroups per head.
-int attention_step(a81w41_qwen3* m, LayerWeights& L, float* out, void* q_out, int splits, float scale, hipStream_t s) {
+int attention_step(a81w41_qwen3* m, LayerWeights& L, float* out, void* q_out, int splits, float scale, hipStream_t s,
+                   const a81w41::ChainLink* link) {
     const a81w41_qwen3_config& c = m->cfg;
     if (splits <= 1)
         Q_HIP(a81w41::launch_attention_one_token(m->qkv, c.n_q_heads, c.n_kv_heads, L.norm[2], L.norm[3], m->cos_t, m->sin_t,
-                                                 m->pos, L.k_cache, L.v_cache, out, q_out, c.max_seq, c.rms_eps, scale, s));
+                                                 m->pos, L.k_cache, L.v_cache, out, q_out, c.max_seq, c.rms_eps, scale, s, link));
     else
         Q_HIP(a81w41::launch_attention_one_token_split(m->qkv, c.n_q_heads, c.n_kv_heads, L.norm[2], L.norm[3], m->cos_t,
                                                        m->sin_t, m->pos, L.k_cache, L.v_cache, out, q_out, m->attn_part,
-                                                       m->attn_arrive, splits, c.max_seq, c.rms_eps, scale, s));
+                                                       m->attn_arrive, splits, c.max_seq, c.rms_eps, scale, s, link));
     return 0;
 }
 
@@ -220,6 +222,28 @@ int enqueue_pass_one_token(a81w41_qwen3* m, hipStream_t s) {
     if (env_split > 0) splits = env_split;
     splits = splits < 1 ? 1 : (splits > a81w41::kAttentionMaxSplits ? a81w41::kAttentionMaxSplits : splits);
     Q_HIP(a81w41::launch_embed_rows(m->ids, m->embedding, m->o, 1, c.hidden, c.vocab, s));  // pending = the embedding
+    // The linears and the attention of the pass are one dependent chain (QwenDecoderLayer.cc:39-105).  As links of
+    // an overlapping chain each of them starts while its predecessor runs and requests its first weight blocks
+    // (or cache rows) before it waits for it; same kernels' arithmetic, same bits.
+    a81w41::ChainState* chain = nullptr;
+    if (m->opt_chain && !no_pair && a81w41::gemv_chain_fits(c.hidden, true) && a81w41::gemv_chain_fits(c.intermediate, false) &&
+        a81w41::gemv_chain_fits(c.n_q_heads * kHeadDim, false))
+        chain = a81w41::context_chain(m->ctx);
+    if (chain) {
+        chain->spin_limit = m->opt_spin_limit ? m->opt_spin_limit : a81w41::ChainState{}.spin_limit;
+        Q_HIP(a81w41::chain_begin(chain, s));
+    }
+    struct CloseOnExit {  // a failed launch must not leave the chain open (and the side stream forked)
+        a81w41::ChainState* c;
+        ~CloseOnExit() {
+            if (c && c->open) (void)a81w41::chain_end(c);
+        }
+    } close_on_exit{chain};
+    // every launch of the chained pass: the link and stream it gets, and the workgroups the next link waits for
+    hipStream_t ls = s;
+    a81w41::ChainLink link;
+    unsigned grid = 0;
+    auto next_link = [&]() { link = a81w41::chain_next(chain, &ls); };
     const float* res_in = nullptr;
     for (int l = 0; l < c.n_layers; l++) {
         LayerWeights& L = m->layers[l];
@@ -228,22 +252,52 @@ int enqueue_pass_one_token(a81w41_qwen3* m, hipStream_t s) {
         p0.res_out = m->x2;
         p0.norm_w = L.norm[0];
         p0.eps = c.rms_eps;
-        Q_HIP(a81w41::launch_gemv_add_norm(m->o, p0, scratch, a81w41_linear_weight_fp16_dev(L.lin[0]), m->qkv, qkv_dim,
-                                           c.hidden, s));
-        if (attn_fp32) {
-            Q_TRY(attention_step(m, L, m->attn, nullptr, splits, scale, s));
-            Q_TRY(a81w41_linear_forward(L.lin[1], m->attn, 1, m->o, s));
-        } else {  // the attention kernel hands o_proj its input already quantised
-            Q_TRY(attention_step(m, L, nullptr, scratch, splits, scale, s));
-            Q_HIP(a81w41::launch_gemv_fp16(scratch, a81w41_linear_weight_fp16_dev(L.lin[1]), m->o, c.hidden,
-                                           c.n_q_heads * kHeadDim, s));
+        if (chain) {
+            next_link();
+            Q_HIP(a81w41::launch_gemv_chain_add_norm(m->o, p0, scratch, a81w41_linear_weight_fp16_dev(L.lin[0]), m->qkv, qkv_dim,
+                                                     c.hidden, link, chain->cus, &grid, ls));
+            a81w41::chain_launched(chain, grid);
+            next_link();
+            Q_TRY(attention_step(m, L, attn_fp32 ? m->attn : nullptr, attn_fp32 ? nullptr : scratch, splits, scale, ls, &link));
+            a81w41::chain_launched(chain, (unsigned)(c.n_q_heads * splits));
+            next_link();
+            if (attn_fp32) {
+                const void* B = a81w41_linear_weight_fp16_dev(L.lin[1]);
+                Q_HIP(a81w41::launch_gemv_chain_fused(m->attn, scratch, 1, &B, &m->o, &c.hidden, c.n_q_heads * kHeadDim, link,
+                                                      chain->cus, &grid, ls));
+            } else {
+                Q_HIP(a81w41::launch_gemv_chain_blob(scratch, a81w41_linear_weight_fp16_dev(L.lin[1]), m->o, c.hidden,
+                                                     c.n_q_heads * kHeadDim, link, chain->cus, &grid, ls));
+            }
+            a81w41::chain_launched(chain, grid);
+        } else {
+            Q_HIP(a81w41::launch_gemv_add_norm(m->o, p0, scratch, a81w41_linear_weight_fp16_dev(L.lin[0]), m->qkv, qkv_dim,
+                                               c.hidden, s));
+            if (attn_fp32) {
+                Q_TRY(attention_step(m, L, m->attn, nullptr, splits, scale, s, nullptr));
+                Q_TRY(a81w41_linear_forward(L.lin[1], m->attn, 1, m->o, s));
+            } else {  // the attention kernel hands o_proj its input already quantised
+                Q_TRY(attention_step(m, L, nullptr, scratch, splits, scale, s, nullptr));
+                Q_HIP(a81w41::launch_gemv_fp16(scratch, a81w41_linear_weight_fp16_dev(L.lin[1]), m->o, c.hidden,
+                                               c.n_q_heads * kHeadDim, s));
+            }
         }
         a81w41::GemvPrologue p1;
         p1.res_in = m->x2;
         p1.res_out = m->x;
         p1.norm_w = L.norm[1];
         p1.eps = c.rms_eps;
-        if (no_pair) {
+        if (chain) {  // gate_up writes silu(gate) * up as quantised blocks: down_proj's input, ready to contract
+            p1.pair_out = static_cast<uint8_t*>(scratch);
+            next_link();
+            Q_HIP(a81w41::launch_gemv_chain_add_norm_silu_pair(m->o, p1, a81w41_linear_weight_fp16_dev(L.lin[2]),
+                                                               2 * c.intermediate, c.hidden, link, chain->cus, &grid, ls));
+            a81w41::chain_launched(chain, grid);
+            next_link();
+            Q_HIP(a81w41::launch_gemv_chain_blob(scratch, a81w41_linear_weight_fp16_dev(L.lin[3]), m->o, c.hidden, c.intermediate,
+                                                 link, chain->cus, &grid, ls));
+            a81w41::chain_launched(chain, grid);
+        } else if (no_pair) {
             Q_HIP(a81w41::launch_gemv_add_norm(m->o, p1, scratch, a81w41_linear_weight_fp16_dev(L.lin[2]), m->gate_up,
                                                2 * c.intermediate, c.hidden, s));
             Q_HIP(a81w41::launch_gemv_silu_mul(m->gate_up, scratch, a81w41_linear_weight_fp16_dev(L.lin[3]), m->o, c.hidden,
@@ -261,8 +315,16 @@ int enqueue_pass_one_token(a81w41_qwen3* m, hipStream_t s) {
     pf.res_out = m->x2;
     pf.norm_w = m->final_norm;
     pf.eps = c.rms_eps;
-    Q_HIP(a81w41::launch_gemv_add_norm(m->o, pf, scratch, a81w41_linear_weight_fp16_dev(m->lm_head), m->logits, c.vocab,
-                                       c.hidden, s));
+    if (chain) {
+        next_link();
+        Q_HIP(a81w41::launch_gemv_chain_add_norm(m->o, pf, scratch, a81w41_linear_weight_fp16_dev(m->lm_head), m->logits, c.vocab,
+                                                 c.hidden, link, chain->cus, &grid, ls));
+        a81w41::chain_launched(chain, grid);
+        Q_HIP(a81w41::chain_end(chain));
+    } else {
+        Q_HIP(a81w41::launch_gemv_add_norm(m->o, pf, scratch, a81w41_linear_weight_fp16_dev(m->lm_head), m->logits, c.vocab,
+                                           c.hidden, s));
+    }
     Q_HIP(a81w41::launch_advance(m->pos, 1, s));
     return 0;
 }
@@ -282,6 +344,18 @@ bool one_token_pass_usable(const a81w41_qwen3* m) {
         for (int w = 0; w < 4; w++)
             if (!a81w41_linear_weight_fp16_dev(L.lin[w])) return false;
     return a81w41_linear_weight_fp16_dev(m->lm_head) != nullptr;
+}
+
+// After a synchronisation: did an in-kernel wait of a chained pass give up?  (Clears the condition.)
+int check_chain(a81w41_qwen3* m) {
+    a81w41::ChainState* chain = a81w41::context_chain(m->ctx);
+    if (!chain || chain->open) return 0;
+    bool gave_up = false;
+    Q_HIP(a81w41::chain_status(chain, &gave_up));
+    if (gave_up)
+        return fail(A81W41_ERR_HIP, "a wait inside the chained one-token pass gave up: the results of that pass are invalid "
+                                    "(is the GPU shared with other work?)");
+    return 0;
 }
 
 template <typename T>
@@ -442,6 +516,11 @@ int a81w41_qwen3_set_option(a81w41_qwen3* m, int option, int value) {
         case A81W41_QWEN3_OPT_ATTN_FP32: m->opt_attn_fp32 = value != 0; break;
         case A81W41_QWEN3_OPT_NO_PAIR: m->opt_no_pair = value != 0; break;
         case A81W41_QWEN3_OPT_VECTOR_ATTENTION: m->opt_vector_attention = value != 0; break;
+        case A81W41_QWEN3_OPT_CHAIN: m->opt_chain = value != 0; break;
+        case A81W41_QWEN3_OPT_CHAIN_SPIN_LIMIT:
+            if (value < 0) return fail(A81W41_ERR_INVALID_ARG, "spin limit must be >= 0 (0: default)");
+            m->opt_spin_limit = (unsigned)value;
+            break;
         case A81W41_QWEN3_OPT_ATTENTION_SPLIT:
             if (value < 0 || value > a81w41::kAttentionMaxSplits)
                 return fail(A81W41_ERR_INVALID_ARG, "attention split must be 0 (automatic) .. %d", a81w41::kAttentionMaxSplits);
@@ -450,6 +529,12 @@ int a81w41_qwen3_set_option(a81w41_qwen3* m, int option, int value) {
         default: return fail(A81W41_ERR_INVALID_ARG, "unknown option %d", option);
     }
     return A81W41_OK;
+}
+
+int a81w41_qwen3_chain_status(a81w41_qwen3* m, int* gave_up) {
+    if (!m || !gave_up) return fail(A81W41_ERR_INVALID_ARG, "null argument");
+    Q_HIP(hipStreamSynchronize(m->stream));
+    return a81w41_context_chain_status(m->ctx, gave_up);
 }
 
 int a81w41_qwen3_read_buffer(a81w41_qwen3* m, int which, float* host_out, size_t count) {
@@ -494,6 +579,7 @@ int a81w41_qwen3_forward(a81w41_qwen3* m, const int* token_ids, int n_tokens, fl
     Q_TRY(enqueue_pass(m, n_tokens, m->stream));
     Q_HIP(hipStreamSynchronize(m->stream));
     m->host_pos += n_tokens;
+    Q_TRY(check_chain(m));
     if (logits_host) Q_HIP(hipMemcpy(logits_host, m->logits, (size_t)m->cfg.vocab * 4, hipMemcpyDeviceToHost));
     return A81W41_OK;
 }
@@ -622,6 +708,7 @@ int a81w41_qwen3_generate_greedy(a81w41_qwen3* m, const int* prompt, int n_promp
     if (n_steps > 0) Q_HIP(hipEventElapsedTime(&ms12, e3, e2));
     if (prefill_ms) *prefill_ms = ms01;
     if (decode_ms) *decode_ms = ms12;
+    Q_TRY(check_chain(m));
     Q_HIP(hipMemcpy(out_tokens, m->history, (size_t)n_new * sizeof(int), hipMemcpyDeviceToHost));
     return A81W41_OK;
 }

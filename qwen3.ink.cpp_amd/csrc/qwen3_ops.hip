@@ -476,13 +476,17 @@ __device__ __forceinline__ void fold_waves(const float* part, const float* wm, c
 // rounded to fp16 as the cache holds them, used from LDS as the last row of the context, and
 // written to the cache by the first query head of the group only.  Rows 0..pos-1 come from the
 // cache, so no workgroup reads what another one writes.
+// CHAIN: the launch is a link of a chain of overlapping launches (chain.h): the norm weights, the rotation and
+// the first cached rows are requested first, then the workgroup waits for the launch that writes qkv, reads the
+// new token's row with agent-scope loads, and its outputs leave with agent-scope stores before it signals.
+template <bool CHAIN>
 __global__ __launch_bounds__(1024) void attention_one_token_kernel(const float* __restrict__ qkv, int n_q, int n_kv,
                                                                  const float* __restrict__ q_w, const float* __restrict__ k_w,
                                                                  const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                                                  const int* __restrict__ pos_dev, __half* __restrict__ k_cache,
                                                                  __half* __restrict__ v_cache, float* __restrict__ out,
                                                                  uint8_t* __restrict__ q_out, int max_seq, float eps,
-                                                                 float scale) {
+                                                                 float scale, const ChainLink link) {
     constexpr int kWaves = 16;
     extern __shared__ float sm[];  // [0, kWaves*128): the waves' weighted values; 3*128: q, new key, new value
     __shared__ float wm[kWaves], wl[kWaves];
@@ -501,11 +505,14 @@ __global__ __launch_bounds__(1024) void attention_one_token_kernel(const float* 
     // lane requests its first cached key rows, whose round trip then overlaps the prepare step; the
     // barriers from here to the weighting step order LDS only, so requested rows stay in flight.
     float x0 = 0.f, x1 = 0.f, w0 = 0.f, w1 = 0.f, c0 = 0.f, c1 = 0.f, s0 = 0.f, s1 = 0.f;
+    const float* src = nullptr;
     if (wave < 3) {
         const int src_head = wave == 0 ? head : (wave == 1 ? n_q + kvh : n_q + n_kv + kvh);
-        const float* src = qkv + (size_t)src_head * kHeadDim;
-        x0 = src[lane];
-        x1 = src[lane + 64];
+        src = qkv + (size_t)src_head * kHeadDim;
+        if (!CHAIN) {
+            x0 = src[lane];
+            x1 = src[lane + 64];
+        }
         if (wave < 2) {
             const float* w = wave == 0 ? q_w : k_w;
             const float* c = cos_t + (size_t)pos * kHeadDim;
@@ -518,6 +525,14 @@ __global__ __launch_bounds__(1024) void attention_one_token_kernel(const float* 
     uint4 k_first[kRowsAhead], v_first[kRowsAhead];
     load_first_rows<kWaves, kRowsAhead>(K4, pos, 4 * wave + grp, k_first);
     load_first_rows<kWaves, kRowsAhead>(V4, pos, 4 * wave + grp, v_first);
+    if (CHAIN) {
+        __builtin_amdgcn_sched_barrier(0);
+        chain_wait(link);
+        if (wave < 3) {
+            x0 = load_agent(src + lane);
+            x1 = load_agent(src + lane + 64);
+        }
+    }
     if (wave == 2) {
         const __half h0 = __float2half_rn(x0), h1 = __float2half_rn(x1);
         v_new[lane] = __half2float(h0);
@@ -565,10 +580,13 @@ __global__ __launch_bounds__(1024) void attention_one_token_kernel(const float* 
         // the head's 128 outputs are four whole 32-blocks of the row: with q_out they go out as the
         // quantised blocks the next linear's quantiser would make of them
         if (q_out != nullptr)
-            store_quantized_value_fp16(q_out, head * kHeadDim + t, val);
+            store_quantized_value_fp16<CHAIN>(q_out, head * kHeadDim + t, val);
+        else if (CHAIN)
+            store_agent(out + (size_t)head * kHeadDim + t, val);
         else
             out[(size_t)head * kHeadDim + t] = val;
     }
+    if (CHAIN) chain_signal(link, gridDim.x);
 }
 
 // The same step for long contexts: S workgroups per query head, workgroup (head, s) takes the cached
@@ -579,11 +597,12 @@ __global__ __launch_bounds__(1024) void attention_one_token_kernel(const float* 
 // are accessed with agent-scope relaxed atomics only (coherent across the XCDs' L2s on their own) and
 // ordered by waiting for the stores and by the workgroup barriers.
 constexpr int kSplitStride = 132;
+template <bool CHAIN>
 __global__ __launch_bounds__(1024) void attention_one_token_split_kernel(
     const float* __restrict__ qkv, int n_q, int n_kv, const float* __restrict__ q_w, const float* __restrict__ k_w,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t, const int* __restrict__ pos_dev,
     __half* __restrict__ k_cache, __half* __restrict__ v_cache, float* __restrict__ out, uint8_t* __restrict__ q_out,
-    float* __restrict__ partials, unsigned* __restrict__ arrivals, int max_seq, float eps, float scale) {
+    float* __restrict__ partials, unsigned* __restrict__ arrivals, int max_seq, float eps, float scale, const ChainLink link) {
     constexpr int kWaves = 16;
     extern __shared__ float sm[];  // [0, kWaves*128): the waves' weighted values; 3*128: q, new key, new value
     __shared__ float wm[kWaves], wl[kWaves];
@@ -605,11 +624,14 @@ __global__ __launch_bounds__(1024) void attention_one_token_split_kernel(
     // as in the one-workgroup kernel: prepare loads, then the first key rows, LDS-only barriers up to the weighting
     const bool prepares = wave == 0 || (own && wave < 3);
     float x0 = 0.f, x1 = 0.f, w0 = 0.f, w1 = 0.f, c0 = 0.f, c1 = 0.f, s0 = 0.f, s1 = 0.f;
+    const float* src = nullptr;
     if (prepares) {
         const int src_head = wave == 0 ? head : (wave == 1 ? n_q + kvh : n_q + n_kv + kvh);
-        const float* src = qkv + (size_t)src_head * kHeadDim;
-        x0 = src[lane];
-        x1 = src[lane + 64];
+        src = qkv + (size_t)src_head * kHeadDim;
+        if (!CHAIN) {
+            x0 = src[lane];
+            x1 = src[lane + 64];
+        }
         if (wave < 2) {
             const float* w = wave == 0 ? q_w : k_w;
             const float* c = cos_t + (size_t)pos * kHeadDim;
@@ -622,6 +644,14 @@ __global__ __launch_bounds__(1024) void attention_one_token_split_kernel(
     uint4 k_first[kRowsAhead], v_first[kRowsAhead];
     load_first_rows<kWaves, kRowsAhead>(K4, n, 4 * wave + grp, k_first);
     load_first_rows<kWaves, kRowsAhead>(V4, n, 4 * wave + grp, v_first);
+    if (CHAIN) {
+        __builtin_amdgcn_sched_barrier(0);
+        chain_wait(link);
+        if (prepares) {
+            x0 = load_agent(src + lane);
+            x1 = load_agent(src + lane + 64);
+        }
+    }
     if (prepares && wave == 2) {
         const __half h0 = __float2half_rn(x0), h1 = __float2half_rn(x1);
         v_new[lane] = __half2float(h0);
@@ -676,7 +706,10 @@ __global__ __launch_bounds__(1024) void attention_one_token_split_kernel(
     __syncthreads();
     if (t == 0) s_arrived = atomicAdd(&arrivals[head], 1u);
     __syncthreads();
-    if (s_arrived != (unsigned)(S - 1)) return;
+    if (s_arrived != (unsigned)(S - 1)) {
+        if (CHAIN) chain_signal(link, gridDim.x * gridDim.y);
+        return;
+    }
     if (t < kHeadDim) {
         const float* base = partials + (size_t)head * S * kSplitStride;
         float m_all = -3.402823466e38f;
@@ -690,11 +723,14 @@ __global__ __launch_bounds__(1024) void attention_one_token_split_kernel(
         }
         const float val = o_all / l_all;
         if (q_out != nullptr)
-            store_quantized_value_fp16(q_out, head * kHeadDim + t, val);
+            store_quantized_value_fp16<CHAIN>(q_out, head * kHeadDim + t, val);
+        else if (CHAIN)
+            store_agent(out + (size_t)head * kHeadDim + t, val);
         else
             out[(size_t)head * kHeadDim + t] = val;
     }
     if (t == 0) __hip_atomic_store(&arrivals[head], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+    if (CHAIN) chain_signal(link, gridDim.x * gridDim.y);
 }
 
 // out[m][j] = silu(gate_up[m][j]) * gate_up[m][inter + j]
@@ -845,22 +881,34 @@ hipError_t launch_attention(const float* q, int q_row_stride, const void* k_cach
 
 hipError_t launch_attention_one_token(const float* qkv, int n_q, int n_kv, const float* q_w, const float* k_w,
                                       const float* cos_t, const float* sin_t, const int* pos_dev, void* k_cache, void* v_cache,
-                                      float* out, void* q_out, int max_seq, float eps, float scale, hipStream_t s) {
+                                      float* out, void* q_out, int max_seq, float eps, float scale, hipStream_t s,
+                                      const ChainLink* link) {
     const size_t lds = (size_t)(16 * kHeadDim + 3 * kHeadDim) * sizeof(float);
-    hipLaunchKernelGGL(attention_one_token_kernel, dim3(n_q), dim3(1024), lds, s, qkv, n_q, n_kv, q_w, k_w, cos_t, sin_t, pos_dev,
-                       static_cast<__half*>(k_cache), static_cast<__half*>(v_cache), out, static_cast<uint8_t*>(q_out), max_seq,
-                       eps, scale);
+    if (link)
+        hipLaunchKernelGGL(attention_one_token_kernel<true>, dim3(n_q), dim3(1024), lds, s, qkv, n_q, n_kv, q_w, k_w, cos_t, sin_t,
+                           pos_dev, static_cast<__half*>(k_cache), static_cast<__half*>(v_cache), out,
+                           static_cast<uint8_t*>(q_out), max_seq, eps, scale, *link);
+    else
+        hipLaunchKernelGGL(attention_one_token_kernel<false>, dim3(n_q), dim3(1024), lds, s, qkv, n_q, n_kv, q_w, k_w, cos_t, sin_t,
+                           pos_dev, static_cast<__half*>(k_cache), static_cast<__half*>(v_cache), out,
+                           static_cast<uint8_t*>(q_out), max_seq, eps, scale, ChainLink{});
     return hipGetLastError();
 }
 
 hipError_t launch_attention_one_token_split(const float* qkv, int n_q, int n_kv, const float* q_w, const float* k_w,
                                             const float* cos_t, const float* sin_t, const int* pos_dev, void* k_cache,
                                             void* v_cache, float* out, void* q_out, float* partials, unsigned* arrivals,
-                                            int splits, int max_seq, float eps, float scale, hipStream_t s) {
+                                            int splits, int max_seq, float eps, float scale, hipStream_t s,
+                                            const ChainLink* link) {
     const size_t lds = (size_t)(16 * kHeadDim + 3 * kHeadDim) * sizeof(float);
-    hipLaunchKernelGGL(attention_one_token_split_kernel, dim3(n_q, splits), dim3(1024), lds, s, qkv, n_q, n_kv, q_w, k_w, cos_t,
-                       sin_t, pos_dev, static_cast<__half*>(k_cache), static_cast<__half*>(v_cache), out,
-                       static_cast<uint8_t*>(q_out), partials, arrivals, max_seq, eps, scale);
+    if (link)
+        hipLaunchKernelGGL(attention_one_token_split_kernel<true>, dim3(n_q, splits), dim3(1024), lds, s, qkv, n_q, n_kv, q_w, k_w,
+                           cos_t, sin_t, pos_dev, static_cast<__half*>(k_cache), static_cast<__half*>(v_cache), out,
+                           static_cast<uint8_t*>(q_out), partials, arrivals, max_seq, eps, scale, *link);
+    else
+        hipLaunchKernelGGL(attention_one_token_split_kernel<false>, dim3(n_q, splits), dim3(1024), lds, s, qkv, n_q, n_kv, q_w, k_w,
+                           cos_t, sin_t, pos_dev, static_cast<__half*>(k_cache), static_cast<__half*>(v_cache), out,
+                           static_cast<uint8_t*>(q_out), partials, arrivals, max_seq, eps, scale, ChainLink{});
     return hipGetLastError();
 }
 

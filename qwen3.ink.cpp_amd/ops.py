@@ -219,6 +219,23 @@ class Context:
             raise RuntimeError(f"hipMemcpy failed with {rc}")
         return out
 
+    def chain_begin(self):
+        """Until ``chain_end`` the one-row forward calls of this context's layers (on the current stream) are
+        links of a chain of overlapping launches (``a81w41_context_chain_begin``)."""
+        capi.check(capi.lib().a81w41_context_chain_begin(self.handle, _stream()))
+
+    def chain_end(self):
+        capi.check(capi.lib().a81w41_context_chain_end(self.handle))
+
+    def chain_gave_up(self) -> bool:
+        """Synchronises; whether an in-kernel wait of a chain gave up since the last call (and clears it)."""
+        flag = C.c_int(0)
+        capi.check(capi.lib().a81w41_context_chain_status(self.handle, C.byref(flag)))
+        return bool(flag.value)
+
+    def chain_set_spin_limit(self, polls: int):
+        capi.check(capi.lib().a81w41_context_chain_set_spin_limit(self.handle, int(polls)))
+
     def __del__(self):
         h, self.handle = getattr(self, "handle", None), None
         if h and capi is not None:  # module globals are gone at interpreter shutdown
@@ -365,11 +382,18 @@ class Qwen3Model:
         assert t.shape == (self.cfg.vocab, self.cfg.hidden)
         capi.check(capi.lib().a81w41_qwen3_set_embedding(self.handle, t.ctypes.data))
 
-    OPTIONS = {"unfused": 0, "attn_fp32": 1, "no_pair": 2, "vector_attention": 3, "attention_split": 4}
+    OPTIONS = {"unfused": 0, "attn_fp32": 1, "no_pair": 2, "vector_attention": 3, "attention_split": 4, "chain": 5,
+               "chain_spin_limit": 6}
 
     def set_option(self, name: str, value: int):
         """Test switch of ``a81w41_qwen3_set_option`` (see include/a81w41.h)."""
         capi.check(capi.lib().a81w41_qwen3_set_option(self.handle, self.OPTIONS[name], int(value)))
+
+    def chain_gave_up(self) -> bool:
+        """Synchronises; whether a wait inside a chained one-token pass gave up since the last call (and clears it)."""
+        flag = C.c_int(0)
+        capi.check(capi.lib().a81w41_qwen3_chain_status(self.handle, C.byref(flag)))
+        return bool(flag.value)
 
     BUFFERS = {"residual": 0, "normed": 1, "qkv": 2, "attention": 3, "block_out": 4, "gate_up": 5, "act": 6, "logits": 7}
 

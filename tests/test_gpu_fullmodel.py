@@ -79,6 +79,15 @@ def test_greedy_generation_graph_equals_eager_and_does_not_collapse(full):
     assert toks.tolist() == eager
     assert len(set(eager)) > n_new // 2, eager
     assert t_pre > 0 and t_dec > 0
+    # the same generation with the decode steps as chains of overlapping launches
+    model.set_option("chain", 1)
+    try:
+        model.reset()
+        chained, _, _ = model.generate_greedy(host["prompt"], n_new)
+    finally:
+        model.set_option("chain", 0)
+    assert np.array_equal(toks, chained)
+    assert not model.chain_gave_up()
 
 
 def _passes(model, host, option=None, value=1):
@@ -101,8 +110,10 @@ def test_fusions_are_bit_identical_at_full_size(full):
     model, host = full
     base = _passes(model, host)
     assert np.isfinite(base).all()
-    for opt in ("attn_fp32", "no_pair"):
+    # chain: the one-token pass as a chain of overlapping launches instead of plain launches on one stream
+    for opt in ("attn_fp32", "no_pair", "chain"):
         assert np.array_equal(base, _passes(model, host, opt)), opt
+    assert not model.chain_gave_up()
     # all separate kernels: the prompt pass has the same bits; the one-token passes then run the few-row vector
     # attention instead of the online-softmax kernel, which is another summation order
     unf = _passes(model, host, "unfused")

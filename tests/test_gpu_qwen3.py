@@ -170,6 +170,36 @@ def test_attention_quantised_output_is_bit_identical(models):
     assert np.array_equal(here, _logits_with_option(gpu, "attn_fp32", 1, passes))
 
 
+def test_chained_one_token_pass_is_bit_identical(models):
+    """With the switch on, the one-token pass runs its linears and attention as a chain of overlapping launches
+    instead of plain launches on one stream.  Same kernels' arithmetic in the same order: same logits, eagerly
+    and from the captured graph, also with the attention's fp32 output and with a split context."""
+    gpu, _ = models
+    passes = [[5, 6, 7, 300, 12, 99, 41], [17], [230], [8], [8], [444], [1]]
+    gpu.reset()
+    here = np.stack([gpu.forward(ids) for ids in passes])
+    assert np.array_equal(here, _logits_with_option(gpu, "chain", 1, passes))
+    for opt, val in (("attn_fp32", 1), ("attention_split", 3)):
+        gpu.set_option(opt, val)
+        try:
+            gpu.reset()
+            a = np.stack([gpu.forward(ids) for ids in passes])
+            assert np.array_equal(a, _logits_with_option(gpu, "chain", 1, passes)), opt
+        finally:
+            gpu.set_option(opt, 0)
+    gpu.reset()
+    toks, _, _ = gpu.generate_greedy(passes[0], 12)
+    gpu.set_option("chain", 1)
+    try:
+        gpu.reset()
+        chained, _, _ = gpu.generate_greedy(passes[0], 12)
+    finally:
+        gpu.set_option("chain", 0)
+        gpu.reset()
+    assert np.array_equal(toks, chained)
+    assert not gpu.chain_gave_up()
+
+
 def test_long_prompt_in_two_chunks(pkg, synth, ora):
     """150 tokens, then 45 more on top of the cached context: several query and key tiles of the
     matrix-core attention, the causal mask inside and across tiles, and a ragged last tile."""
