@@ -209,11 +209,23 @@ const void *a81w41_linear_weight_fp32_dev(const a81w41_linear *layer);
  * dispatch -- M == 1: fp16-parameter quantiser + GEMV on the 320 B blob,
  * M > 1: fp32-parameter quantiser + GEMM on the 384 B blob.  Device pointers. */
 int a81w41_linear_forward(a81w41_linear *layer, const float *x_dev, int M, float *y_dev, void *stream);
+/* The contraction half of forward for M > 1 (QwenOperator.cc:104-108: the gemm_repack_A81W41_fp32
+ * call on the context's buffer): rows that are already quantised, M*K/64 blocks of 80 B, 16-byte
+ * aligned, contracted by whichever kernel the layer's forward would pick for M rows.  For callers
+ * whose producer writes quantised blocks itself (as the model's norm, SiLU and attention epilogues
+ * do), and for tests that need hand-made int8 rows. */
+int a81w41_linear_forward_quantized(a81w41_linear *layer, const void *a_blob_dev, int M, float *y_dev,
+                                    void *stream);
 /* Which kernel M > 32 calls of this layer contract on.  The layer keeps, beside
  * the reference's two blobs, its fp32-parameter weights in the operand format of
  * gfx950's block-scaled matrix op (exact for these integers, twice the int8
  * rate); by default a call goes there when its shape is one where that kernel is
- * the faster one (A81W41_KERNEL_AUTO).  The other two values exist for tests and
+ * the faster one (A81W41_KERNEL_AUTO).  Its block dots are the reference's
+ * integers bit for bit; its min terms fma(mW, sA, acc) are formed from bf16
+ * pieces (sA exactly, as three; mW as two, i.e. to 16 significant bits, exact
+ * for mins taken from bf16 or fp16 weights), so a call on that kernel agrees
+ * with the int8 kernels to about 2e-5 of the row norm where they agree with
+ * the reference to 1e-6 (the bar of the path is 1e-4).  The other two values exist for tests and
  * measurements: NEVER keeps every call on the int8 kernels, ALWAYS sends every
  * call of more than 32 rows to the block-scaled one.  No counterpart in the
  * reference, which has one kernel per precision (quantized_gemx_kernels.cc:349). */

@@ -50,6 +50,7 @@ SIGNATURES = {
     "a81w41_linear_weight_fp16_dev": (_vp, [_vp]),
     "a81w41_linear_weight_fp32_dev": (_vp, [_vp]),
     "a81w41_linear_forward": (_i, [_vp, _vp, _i, _vp, _vp]),
+    "a81w41_linear_forward_quantized": (_i, [_vp, _vp, _i, _vp, _vp]),
     "a81w41_linear_set_kernel": (_i, [_vp, _i]),
     "a81w41_linear_forward_multi": (_i, [_i, C.POINTER(_vp), _vp, _i, C.POINTER(_vp), _vp]),
     "a81w41_linear_forward_host": (_i, [_vp, _vp, _i, _vp]),

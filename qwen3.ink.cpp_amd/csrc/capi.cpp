@@ -681,6 +681,27 @@ int a81w41_linear_forward(a81w41_linear* l, const float* x_dev, int M, float* y_
     return a81w41_gemv_repack_A81W41_fp16(ctx->act_scratch, l->w16, y_dev, M, l->N, l->K, stream);
 }
 
+int a81w41_linear_forward_quantized(a81w41_linear* l, const void* a_blob_dev, int M, float* y_dev, void* stream) {
+    if (!l || !a_blob_dev || !y_dev) return fail(A81W41_ERR_INVALID_ARG, "null pointer");
+    if (M < 2) return fail(A81W41_ERR_INVALID_ARG, "M must be >= 2 (80 B blocks are the M > 1 format), got %d", M);
+    if (!l->w32) return fail(A81W41_ERR_INVALID_ARG, "layer has no fp32-parameter blob (needed for M > 1)");
+    a81w41_context* ctx = l->ctx;
+    if ((int64_t)M * l->K > ctx->max_elems)
+        return fail(A81W41_ERR_INVALID_ARG, "M*K = %lld exceeds the context's scratch (%lld)", (long long)M * l->K,
+                    (long long)ctx->max_elems);
+    if (int st = contract_args_ok(a_blob_dev, l->w32, y_dev, M, l->N, l->K)) return st;
+    if (reinterpret_cast<uintptr_t>(a_blob_dev) & 15)
+        return fail(A81W41_ERR_INVALID_ARG, "activation blob must be 16-byte aligned");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (a81w41::linear_block_scaled(l, M)) {
+        HIP_TRY(a81w41::launch_a80_to_a6(a_blob_dev, ctx->a6_scratch, M, l->K, s));
+        HIP_TRY(a81w41::launch_gemm_fp6(ctx->a6_scratch, l->w6, y_dev, M, l->N, l->K, ctx->gemm_scratch, s));
+        return A81W41_OK;
+    }
+    HIP_TRY(a81w41::launch_gemm_fp32(a_blob_dev, l->w32, y_dev, M, l->N, l->K, ctx->gemm_scratch, s));
+    return A81W41_OK;
+}
+
 int a81w41_linear_set_kernel(a81w41_linear* l, int choice) {
     if (!l) return fail(A81W41_ERR_INVALID_ARG, "null layer");
     if (choice != A81W41_KERNEL_AUTO && choice != A81W41_KERNEL_INT8 && choice != A81W41_KERNEL_BLOCK_SCALED)

@@ -12,16 +12,19 @@
 // vector ALU (it costs more than the matrix op on this chip, where the two pipes of a SIMD take turns).
 // The rest is the reference's epilogue per (row, column, 32-block), in fp32:
 //   acc = fma(float(idot), fl(dA*dW), acc)       fl(dA*dW): v_mfma_f32_32x32x1_2b_f32 (exact products, one rounding)
-//   acc = fma(mW, sA, acc)                       four 32-blocks at a time on v_mfma_f32_32x32x16_bf16: sA and mW are
-//                                                kept as two bf16 pieces each (hi + lo, 16 significant bits), and
-//                                                hi*hi + hi*lo + lo*hi of a block fill three of the op's 16 K slots.
-//                                                The dropped lo*lo and the pieces' rounding are below 2^-16 of a term.
+//   acc = fma(mW, sA, acc)                       four 32-blocks at a time on v_mfma_f32_32x32x16_bf16: sA is kept as
+//                                                three bf16 pieces (hi + mid + lo = sA exactly), mW as two (16
+//                                                significant bits: exact for mins that come from bf16 or fp16 weights),
+//                                                and s_hi*w_hi + s_hi*w_lo + s_mid*w_hi + s_lo*w_hi of a block fill
+//                                                four of the op's 16 K slots.  Dropped: s_mid*w_lo and s_lo*w_lo, below
+//                                                2^-17 of a term, and nothing at all when mW is a bf16 number.
 //
 // Operand formats (private to the layer object; made once from the reference's blobs):
 //   W6: per (32-column panel, 32-block) 1 KiB: chunk 0 = [32 columns][16 B] fp6 codes k = 0..20 (+2 bits),
 //       chunk 1 = [32 columns][16 B] rest of the codes (8 B), dW (fp32), mW as two bf16 pieces (hi | lo << 16).
 //   A6: per (32-row panel, 32-block) 2 KiB: piece 0 (qh) then piece 1 (ql), each laid out like a W6 panel
-//       with dA (fp32) and the scaled sum sA (two bf16 pieces) in chunk 1.
+//       with dA (fp32) and two of the scaled sum's three bf16 pieces in chunk 1: hi | mid in piece 0's copy, lo in
+//       piece 1's (the two lane halves of the contraction kernel exchange them).
 // A lane reads its operand with two 16-byte loads; lanes of a half-wave read consecutive 16 bytes.
 //
 // Tiling: 128 x 256 tiles of C per workgroup, 8 waves of 64 x 64 (two row panels against two column panels),
@@ -71,6 +74,15 @@ __host__ __device__ __forceinline__ uint32_t split_bf16x2(float x) {
     union { uint32_t u; float f; } h = {hi << 16};
     return hi | (bf16_rne_bits(x - h.f) << 16);  // the subtraction is exact
 }
+// x as three bf16 pieces hi + mid + lo = x exactly (24 significant bits): hi | mid << 16 in .x, lo in .y
+__host__ __device__ __forceinline__ uint2 split_bf16x3(float x) {
+    const uint32_t hi = bf16_rne_bits(x);
+    union { uint32_t u; float f; } h = {hi << 16};
+    const float r1 = x - h.f;  // exact
+    const uint32_t mid = bf16_rne_bits(r1);
+    union { uint32_t u; float f; } m = {mid << 16};
+    return make_uint2(hi | (mid << 16), bf16_rne_bits(r1 - m.f));  // what is left has at most 8 significant bits
+}
 
 // ---- operand preparation ------------------------------------------------------------------------
 
@@ -112,10 +124,14 @@ __device__ __forceinline__ void store_a6_block(uint8_t* __restrict__ a6, int row
         const int piece = j >> 1, chunk = j & 1;
         const uint32_t* dw = piece ? lo : hi;
         uint4 v;
-        if (chunk == 0)
+        if (chunk == 0) {
             v = make_uint4(dw[0], dw[1], dw[2], dw[3]);
-        else
-            v = make_uint4(dw[4], dw[5], __float_as_uint(d), split_bf16x2(ssum));
+        } else {
+            // the scaled sum as three bf16 pieces: hi | mid in the high piece's copy (read by lanes 0..31 of the
+            // contraction kernel), lo in the low piece's copy (lanes 32..63)
+            const uint2 s3 = split_bf16x3(ssum);
+            v = make_uint4(dw[4], dw[5], __float_as_uint(d), piece == 0 ? s3.x : s3.y);
+        }
         uint8_t* dst = a6 + ((size_t)(row >> 5) * nb + blk) * kPanelA + piece * 1024 + chunk * 512 + (row & 31) * 16;
         *reinterpret_cast<uint4*>(dst) = v;
     }
@@ -290,20 +306,23 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         const bool rows_live = kTileM * ty + 64 * wr < M;  // else every row of this wave is past M
 
         // min terms of up to four 32-blocks (zero pieces where the run ends early): lane half 0 brings blocks 0 and 1,
-        // half 1 blocks 2 and 3 (each half keeps only its own two blocks' pieces), three K slots per block:
-        // (s_hi, s_hi, s_lo) against (w_hi, w_lo, w_hi)
-        auto min_terms = [&](const uint32_t (&ya)[2][2], const uint32_t (&yb)[2][2]) {
+        // half 1 blocks 2 and 3, four K slots per block: (s_hi, s_hi, s_mid, s_lo) against (w_hi, w_lo, w_hi, w_hi).
+        // Lanes 0..31 read hi | mid of a scaled sum, lanes 32..63 its lo: ya = this lane's word for the half's own
+        // two blocks, za = its word for the other half's two blocks, which the partner lane (same row, other half)
+        // needs; one exchange per block gives every lane all three pieces of its own blocks.
+        auto min_terms = [&](const uint32_t (&ya)[2][2], const uint32_t (&za)[2][2], const uint32_t (&yb)[2][2]) {
             v4i opa[2], opb[2];
 #pragma unroll
             for (int i = 0; i < 2; i++) {
-                opa[i][0] = (int)__builtin_amdgcn_perm(ya[i][0], ya[i][0], 0x01000100u);  // hi0, hi0
-                opa[i][1] = (int)__builtin_amdgcn_alignbit(ya[i][1], ya[i][0], 16);       // lo0, hi1
-                opa[i][2] = (int)ya[i][1];                                                // hi1, lo1
-                opa[i][3] = 0;
-                opb[i][0] = (int)yb[i][0];                                                // hi0, lo0
-                opb[i][1] = (int)__builtin_amdgcn_perm(yb[i][1], yb[i][0], 0x05040100u);  // hi0, hi1
-                opb[i][2] = (int)__builtin_amdgcn_alignbit(yb[i][1], yb[i][1], 16);       // lo1, hi1
-                opb[i][3] = 0;
+#pragma unroll
+                for (int k = 0; k < 2; k++) {
+                    const uint32_t got = (uint32_t)__shfl_xor((int)za[i][k], 32, 64);
+                    const uint32_t himid = h ? got : ya[i][k], lo = h ? ya[i][k] : got;
+                    opa[i][2 * k] = (int)__builtin_amdgcn_perm(himid, himid, 0x01000100u);  // hi, hi
+                    opa[i][2 * k + 1] = (int)((himid >> 16) | (lo << 16));                       // mid, lo
+                    opb[i][2 * k] = (int)yb[i][k];                                                  // hi, lo
+                    opb[i][2 * k + 1] = (int)__builtin_amdgcn_perm(yb[i][k], yb[i][k], 0x01000100u);  // hi, hi
+                }
             }
             typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
             auto bf = [](const v4i& v) { return __builtin_bit_cast(v8bf, v); };
@@ -337,7 +356,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
             Frag fa[2][2], fb[2][2];  // two sets: the one in use and the next step's, in flight
             load_step(0, fa[0], fb[0]);
             for (int step0 = 0; step0 < n_steps; step0 += 4) {
-                uint32_t ya[2][2] = {{0, 0}, {0, 0}}, yb[2][2] = {{0, 0}, {0, 0}};
+                uint32_t ya[2][2] = {{0, 0}, {0, 0}}, za[2][2] = {{0, 0}, {0, 0}}, yb[2][2] = {{0, 0}, {0, 0}};
 #pragma unroll
                 for (int u4 = 0; u4 < 4; u4++) {
                     const int step = step0 + u4;
@@ -351,10 +370,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                             ya[i][u4 & 1] = (uint32_t)ca[i][7];
                             yb[i][u4 & 1] = (uint32_t)cb[i][7];
                         }
+                    } else {  // the other half's block: the partner lane needs this lane's word of its scaled sums
+#pragma unroll
+                        for (int i = 0; i < 2; i++) za[i][u4 & 1] = (uint32_t)ca[i][7];
                     }
                     compute(ca, cb);
                 }
-                min_terms(ya, yb);
+                min_terms(ya, za, yb);
             }
         }
 

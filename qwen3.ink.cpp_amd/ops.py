@@ -301,6 +301,14 @@ class Linear:
         capi.check(capi.lib().a81w41_linear_forward(self.handle, _dev_ptr(x), M, _dev_ptr(out), _stream()))
         return out
 
+    def forward_quantized(self, a_blob, M: int, out=None):
+        """Rows already quantised (CUDA uint8, M*K/64 blocks of 80 B) -> [M][N] (``a81w41_linear_forward_quantized``)."""
+        torch = _torch()
+        if out is None:
+            out = torch.empty((M, self.N), dtype=torch.float32, device=a_blob.device)
+        capi.check(capi.lib().a81w41_linear_forward_quantized(self.handle, _dev_ptr(a_blob), M, _dev_ptr(out), _stream()))
+        return out
+
     def forward_host(self, x: np.ndarray) -> np.ndarray:
         x = np.ascontiguousarray(x, np.float32)
         M = x.size // self.K
