@@ -91,9 +91,13 @@ int a81w41_gemv_repack_A81W41_fp16(const void *A_repack_dev, const void *B_repac
  * Calls with M > 8 may split the K range of some tiles and park partial tiles in a
  * scratch (64 MiB) that belongs to `stream`: it is allocated by the first such call on
  * that stream (which therefore cannot be captured into a graph; later calls can) and kept
- * until the process ends, at most 16 streams per device.  Calls on one stream are ordered
- * by the stream, calls on different streams use different scratches, so no two launches
- * ever share partial tiles.  Results do not depend on timing. */
+ * until the process ends.  A device keeps at most 16 of them: the first call on a 17th
+ * stream waits for the device to be idle and takes over the scratch of the stream that
+ * used its own longest ago (streams come and go; their scratches are reused).  Calls on one
+ * stream are ordered by the stream, calls on different streams use different scratches, so
+ * no two launches share partial tiles -- with one caveat: a captured graph keeps the
+ * scratch of the stream it was captured on wherever it is replayed, so its replays must
+ * not overlap with K-split calls on that stream.  Results do not depend on timing. */
 int a81w41_gemm_repack_A81W41_fp32(const void *A_repack_dev, const void *B_repack_dev, float *C_dev,
                                    int M, int N, int K, void *stream);
 
@@ -199,6 +203,14 @@ int a81w41_linear_load(a81w41_context *ctx, const char *path, int dim_x, int dim
                        a81w41_linear **out);
 void a81w41_linear_destroy(a81w41_linear *layer);
 
+/* Device memory the layer's weights occupy, in total and per copy: the reference's two blobs
+ * (0.625 and 0.75 B per weight, QwenOperator.h:142-154) and, where the layer has it, the
+ * block-scaled kernel's operand format (1 B per weight).  The third copy exists only for layers
+ * that a call the context admits (max_rows x max_cols) can send to that kernel, or after
+ * a81w41_linear_set_kernel(layer, A81W41_KERNEL_BLOCK_SCALED); A81W41_KERNEL_INT8 frees it.
+ * Out-pointers may be NULL. */
+size_t a81w41_linear_resident_bytes(const a81w41_linear *layer, size_t *fp16_blob, size_t *fp32_blob,
+                                    size_t *block_scaled);
 int a81w41_linear_in_features(const a81w41_linear *layer);  /* K */
 int a81w41_linear_out_features(const a81w41_linear *layer); /* N */
 const void *a81w41_linear_weight_fp16_dev(const a81w41_linear *layer);
@@ -225,9 +237,12 @@ int a81w41_linear_forward_quantized(a81w41_linear *layer, const void *a_blob_dev
  * pieces (sA exactly, as three; mW as two, i.e. to 16 significant bits, exact
  * for mins taken from bf16 or fp16 weights), so a call on that kernel agrees
  * with the int8 kernels to about 2e-5 of the row norm where they agree with
- * the reference to 1e-6 (the bar of the path is 1e-4).  The other two values exist for tests and
- * measurements: NEVER keeps every call on the int8 kernels, ALWAYS sends every
- * call of more than 32 rows to the block-scaled one.  No counterpart in the
+ * the reference to 1e-6 (the bar of the path is 1e-4).  The other two values
+ * exist for tests, measurements and callers short of memory: A81W41_KERNEL_INT8
+ * keeps every call on the int8 kernels and frees the layer's third weight copy,
+ * A81W41_KERNEL_BLOCK_SCALED sends every call of more than 32 rows to the
+ * block-scaled one, building that copy if the layer has none (this allocates and
+ * synchronises: not on a stream that is being captured).  No counterpart in the
  * reference, which has one kernel per precision (quantized_gemx_kernels.cc:349). */
 enum { A81W41_KERNEL_AUTO = 0, A81W41_KERNEL_INT8 = 1, A81W41_KERNEL_BLOCK_SCALED = 2 };
 int a81w41_linear_set_kernel(a81w41_linear *layer, int choice);

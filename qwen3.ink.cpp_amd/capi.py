@@ -45,6 +45,7 @@ SIGNATURES = {
     "a81w41_linear_create_from_blobs": (_i, [_vp, _i, _i, _vp, _vp, C.POINTER(_vp)]),
     "a81w41_linear_load": (_i, [_vp, C.c_char_p, _i, _i, _i, C.POINTER(_vp)]),
     "a81w41_linear_destroy": (None, [_vp]),
+    "a81w41_linear_resident_bytes": (_sz, [_vp, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)]),
     "a81w41_linear_in_features": (_i, [_vp]),
     "a81w41_linear_out_features": (_i, [_vp]),
     "a81w41_linear_weight_fp16_dev": (_vp, [_vp]),

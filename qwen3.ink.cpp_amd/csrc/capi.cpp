@@ -308,9 +308,9 @@ static int stream_scratch(void* stream, int M, int N, int K, a81w41::GemmScratch
     const hipError_t e = a81w41::gemm_scratch_for_stream(static_cast<hipStream_t>(stream), ws);
     if (e == hipErrorStreamCaptureUnsupported)
         return fail(A81W41_ERR_INVALID_ARG,
-                    "the first K-split GEMM call on a stream allocates that stream's scratch and cannot be captured: "
+                    "the first K-split GEMM call on a stream allocates (or takes over) that stream's scratch and cannot be captured: "
                     "call once before the capture, use a layer object, or a81w41_gemm_repack_A81W41_fp32_static");
-    if (e == hipErrorOutOfMemory) return fail(A81W41_ERR_HIP, "GEMM scratch: out of device memory or more than 16 streams");
+    if (e == hipErrorOutOfMemory) return fail(A81W41_ERR_HIP, "GEMM scratch: out of device memory (64 MiB per stream, at most 16 streams' worth)");
     if (e != hipSuccess) return hip_fail(e, "gemm_scratch_for_stream");
     return A81W41_OK;
 }
@@ -468,6 +468,25 @@ void a81w41_context_destroy(a81w41_context* ctx) {
 
 void* a81w41_context_activation_scratch_dev(const a81w41_context* ctx) { return ctx ? ctx->act_scratch : nullptr; }
 
+// The most rows a call of a K-wide layer may have on this context.
+static int max_rows_of(const a81w41_context* ctx, int K) {
+    const int64_t rows = ctx->max_elems / K;
+    return rows > 0x7fffffff ? 0x7fffffff : (int)rows;
+}
+
+// Derives the block-scaled kernel's weight operand from the 384 B blob (on the device, synchronous).
+static hipError_t build_w6(a81w41_linear* l) {
+    if (l->w6 || !l->w32) return hipSuccess;
+    hipError_t e = hipMalloc(&l->w6, a81w41::gemm_fp6_w6_bytes(l->N, l->K));
+    if (e == hipSuccess) e = a81w41::launch_w384_to_w6(l->w32, l->w6, l->N, l->K, nullptr);
+    if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
+    if (e != hipSuccess) {
+        (void)hipFree(l->w6);
+        l->w6 = nullptr;
+    }
+    return e;
+}
+
 int a81w41_linear_create_from_blobs(a81w41_context* ctx, int N, int K, const void* blob_fp16,
                                     const void* blob_fp32, a81w41_linear** out) {
     if (!out) return fail(A81W41_ERR_INVALID_ARG, "null out pointer");
@@ -490,10 +509,9 @@ int a81w41_linear_create_from_blobs(a81w41_context* ctx, int N, int K, const voi
         const size_t b = a81w41_weight_blob_bytes(K, N, 1);
         e = hipMalloc(&l->w32, b);
         if (e == hipSuccess) e = hipMemcpy(l->w32, blob_fp32, b, hipMemcpyHostToDevice);
-        // the operand format of the M > 32 kernel, derived on the device once
-        if (e == hipSuccess) e = hipMalloc(&l->w6, a81w41::gemm_fp6_w6_bytes(N, K));
-        if (e == hipSuccess) e = a81w41::launch_w384_to_w6(l->w32, l->w6, N, K, nullptr);
-        if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
+        // the operand format of the block-scaled kernel (a third copy, 1 B per weight): only where a call this
+        // context admits can be routed there
+        if (e == hipSuccess && a81w41::gemm_fp6_preferred(max_rows_of(ctx, K), N, K)) e = build_w6(l.get());
     }
     if (e != hipSuccess) {
         (void)hipFree(l->w16);
@@ -547,6 +565,17 @@ void a81w41_linear_destroy(a81w41_linear* l) {
     (void)hipFree(l->w32);
     (void)hipFree(l->w6);
     delete l;
+}
+
+size_t a81w41_linear_resident_bytes(const a81w41_linear* l, size_t* fp16_blob, size_t* fp32_blob, size_t* block_scaled) {
+    if (!l) return 0;
+    const size_t b16 = l->w16 ? a81w41_weight_blob_bytes(l->K, l->N, 0) : 0;
+    const size_t b32 = l->w32 ? a81w41_weight_blob_bytes(l->K, l->N, 1) : 0;
+    const size_t b6 = l->w6 ? a81w41::gemm_fp6_w6_bytes(l->N, l->K) : 0;
+    if (fp16_blob) *fp16_blob = b16;
+    if (fp32_blob) *fp32_blob = b32;
+    if (block_scaled) *block_scaled = b6;
+    return b16 + b32 + b6;
 }
 
 int a81w41_linear_in_features(const a81w41_linear* l) { return l ? l->K : 0; }
@@ -706,6 +735,13 @@ int a81w41_linear_set_kernel(a81w41_linear* l, int choice) {
     if (!l) return fail(A81W41_ERR_INVALID_ARG, "null layer");
     if (choice != A81W41_KERNEL_AUTO && choice != A81W41_KERNEL_INT8 && choice != A81W41_KERNEL_BLOCK_SCALED)
         return fail(A81W41_ERR_INVALID_ARG, "unknown kernel choice %d", choice);
+    if (choice == A81W41_KERNEL_INT8) {  // the third weight copy is of no use any more
+        HIP_TRY(hipDeviceSynchronize());
+        (void)hipFree(l->w6);
+        l->w6 = nullptr;
+    } else if (l->w32 && (choice == A81W41_KERNEL_BLOCK_SCALED || a81w41::gemm_fp6_preferred(max_rows_of(l->ctx, l->K), l->N, l->K))) {
+        HIP_TRY(build_w6(l));  // allocates and synchronises: not for a stream that is being captured
+    }
     l->kernel_choice = choice;
     return A81W41_OK;
 }

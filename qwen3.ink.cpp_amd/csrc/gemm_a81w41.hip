@@ -447,7 +447,7 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
 // file-scope array below for the entry point that may not allocate.
 constexpr int kMaxPartials = 4096;  // room for every tile of a launch that does not fill the chip to be cut in four
 constexpr int kMaxDevices = 64;
-constexpr int kMaxStreamsPerDevice = 16;
+constexpr int kMaxStreamsPerDevice = 16;  // scratches kept per device; a further stream takes over the least recently used one
 
 // Static scratch of the allocation-free entry point: 2048 partial tiles (32 MiB) and their counters per
 // device, held from the moment the code object is loaded until the process ends.
@@ -465,8 +465,10 @@ struct DeviceInfo {
     struct {
         hipStream_t stream;
         GemmScratch ws;
+        unsigned long long last_use;
     } by_stream[kMaxStreamsPerDevice];
     int n_streams = 0;
+    unsigned long long uses = 0;
 };
 DeviceInfo g_dev[kMaxDevices];
 std::mutex g_dev_mutex;
@@ -650,19 +652,34 @@ hipError_t gemm_scratch_for_stream(hipStream_t s, GemmScratch* out) {
     if (e != hipSuccess) return e;
     for (int i = 0; i < d->n_streams; i++)
         if (d->by_stream[i].stream == s) {
+            d->by_stream[i].last_use = ++d->uses;
             *out = d->by_stream[i].ws;
             return hipSuccess;
         }
-    if (d->n_streams == kMaxStreamsPerDevice) return hipErrorOutOfMemory;
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     e = hipStreamIsCapturing(s, &cap);
     if (e != hipSuccess) return e;
-    if (cap != hipStreamCaptureStatusNone) return hipErrorStreamCaptureUnsupported;  // cannot allocate under capture
+    if (cap != hipStreamCaptureStatusNone) return hipErrorStreamCaptureUnsupported;  // cannot allocate or wait under capture
+    if (d->n_streams == kMaxStreamsPerDevice) {
+        // Every scratch is taken: the stream that used its own longest ago (it may not even exist any more) hands it
+        // over.  Work that still uses it may be in flight, so the device is drained first; the counters are zero
+        // between launches, so nothing needs clearing.
+        e = hipDeviceSynchronize();
+        if (e != hipSuccess) return e;
+        int lru = 0;
+        for (int i = 1; i < d->n_streams; i++)
+            if (d->by_stream[i].last_use < d->by_stream[lru].last_use) lru = i;
+        d->by_stream[lru].stream = s;
+        d->by_stream[lru].last_use = ++d->uses;
+        *out = d->by_stream[lru].ws;
+        return hipSuccess;
+    }
     GemmScratch ws;
     e = gemm_scratch_create(&ws);
     if (e != hipSuccess) return e;
     d->by_stream[d->n_streams].stream = s;
     d->by_stream[d->n_streams].ws = ws;
+    d->by_stream[d->n_streams].last_use = ++d->uses;
     d->n_streams++;
     *out = ws;
     return hipSuccess;

@@ -301,6 +301,12 @@ class Linear:
         capi.check(capi.lib().a81w41_linear_forward(self.handle, _dev_ptr(x), M, _dev_ptr(out), _stream()))
         return out
 
+    def resident_bytes(self) -> dict:
+        """Device bytes of the layer's weight copies (``a81w41_linear_resident_bytes``)."""
+        a, b, c = C.c_size_t(), C.c_size_t(), C.c_size_t()
+        total = capi.lib().a81w41_linear_resident_bytes(self.handle, C.byref(a), C.byref(b), C.byref(c))
+        return {"total": int(total), "fp16_blob": a.value, "fp32_blob": b.value, "block_scaled": c.value}
+
     def forward_quantized(self, a_blob, M: int, out=None):
         """Rows already quantised (CUDA uint8, M*K/64 blocks of 80 B) -> [M][N] (``a81w41_linear_forward_quantized``)."""
         torch = _torch()
