@@ -7,10 +7,11 @@ One *step* is one decoded token's worth of quantized-linear calls -- 36 layers x
 (activation quantiser + GEMV), each layer with its own resident weights
 (4.73 GB of packed int4 blocks, so every step streams from HBM, not from the
 256 MB last-level cache).  ``value`` is algorithmic bytes per step / wall time
-per step with the launches replayed from a HIP graph.  The 253 calls of the sweep
-are independent of each other, so the graph holds them as parallel branches
-(``--branches``, equal-priority streams forked and joined inside the capture);
-``serial_chain`` is the same step captured as one dependent chain.
+per step with the launches replayed from a HIP graph as ONE dependent chain on one
+stream -- what a decode pass is (every linear waits for the one before it).  The
+253 calls of this synthetic sweep happen to be independent of each other, so the
+same step is also timed with its layers captured as parallel branches
+(``side_by_side``, ``--branches``); that figure is not a rate a model can reach.
 
 Also reported in the same JSON line:
   roofline      the GEMV kernel alone: algorithmic bytes / launch-to-launch time of a
@@ -19,7 +20,9 @@ Also reported in the same JSON line:
   qgemm         the M=322 prefill forward (quantiser + GEMM) over the seven layer
                 shapes, weights rotated over the 36 layers' copies (TOPS)
   m_sweep       forward at M in {1, 8, 32, 128, 512, 2048} on gate and down
-  e2e           random-init Qwen3-8B: 322-token prefill + 128 greedy decode steps
+  e2e           random-init Qwen3-8B: 322-token prefill + 128 greedy decode steps, resident bytes
+  a80w40        the A80W40 variant's GEMV sweep and M=322 GEMM
+Every figure is the median of five timed windows (the minimum is reported beside it).
   cpu_baseline  the AVX2+OpenMP port of the reference's CPU path on this host
 """
 from __future__ import annotations
@@ -60,7 +63,7 @@ def gemv_bytes(K, N):
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--layers", type=int, default=N_LAYERS, help="decoder layers resident (36 = Qwen3-8B)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -89,14 +92,17 @@ def parse():
                     help="also time every shape's GEMV alone, from an already quantised activation blob "
                          "(gemv_repack_A81W41_fp16 as the reference declares it), over the same distinct weight copies "
                          "(extra kernel launches: leave off when the run is profiled)")
-    ap.add_argument("--a80w40", action="store_true",
-                    help="also time the A80W40 variant: its GEMV over the eight shapes (weights rotated through "
+    ap.add_argument("--no-a80w40", action="store_true",
+                    help="skip the A80W40 variant's leg: its GEMV over the eight shapes (weights rotated through "
                          ">= 400 MB of copies) and its M=322 GEMM over the seven layer shapes")
+    ap.add_argument("--no-chain", action="store_true",
+                    help="skip the step as a chain of overlapping launches (a81w41_context_chain_*)")
     args = ap.parse_args()
     if args.profile:
-        args.no_m_sweep = args.no_e2e = args.no_grouped = args.no_cpu = True
+        args.no_m_sweep = args.no_e2e = args.no_grouped = args.no_cpu = args.no_a80w40 = args.no_chain = True
         args.branches = 1
     args.m_sweep, args.e2e, args.grouped = not args.no_m_sweep, not args.no_e2e, not args.no_grouped
+    args.a80w40 = not args.no_a80w40
     return args
 
 
@@ -188,35 +194,101 @@ def main():
         for st in side:
             main.wait_stream(st)
 
+    N_WINDOWS = 5
+
     def time_graph(fn):
+        """Captures fn into a HIP graph; W untimed replays, then N_WINDOWS windows of exactly K replays each,
+        bracketed by synchronisations.  -> (median, minimum) of the windows' milliseconds per replay."""
         fn()                            # eager once (also checks every call)
         stream.synchronize()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=stream):
+        with torch.cuda.graph(graph, stream=stream, capture_error_mode="thread_local"):
             fn()
         for _ in range(args.warmup):
             graph.replay()
+        windows = []
+        for _ in range(N_WINDOWS):
+            stream.synchronize()
+            torch.cuda.synchronize()
+            t_start = time.perf_counter()
+            for _ in range(args.steps):
+                graph.replay()
+            stream.synchronize()
+            torch.cuda.synchronize()
+            windows.append((time.perf_counter() - t_start) * 1e3 / args.steps)
+        return float(np.median(windows)), float(min(windows))
+
+    def time_events(graph, units_per_replay, min_window_ms=40.0):
+        """A captured graph timed with events on the launch stream: N_WINDOWS windows of at least min_window_ms
+        each.  -> (median, minimum) microseconds per unit."""
+        graph.replay()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        graph.replay()
+        e1.record(stream)
         stream.synchronize()
-        torch.cuda.synchronize()
-        t_start = time.perf_counter()
-        for _ in range(args.steps):
-            graph.replay()
+        reps = max(2, int(min_window_ms / max(e0.elapsed_time(e1), 1e-3)) + 1)
+        out = []
+        for _ in range(N_WINDOWS):
+            e0.record(stream)
+            for _ in range(reps):
+                graph.replay()
+            e1.record(stream)
+            stream.synchronize()
+            out.append(e0.elapsed_time(e1) * 1e3 / (reps * units_per_replay))
+        return float(np.median(out)), float(min(out))
+
+    def capture(fn):
+        fn()
         stream.synchronize()
-        torch.cuda.synchronize()
-        return (time.perf_counter() - t_start) * 1e3 / args.steps
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream, capture_error_mode="thread_local"):
+            fn()
+        return g
 
     stream = torch.cuda.Stream()
+    side_by_side = overlapped = None
     with torch.cuda.stream(stream):
-        ms_chain = time_graph(run_step)
+        ms_per_step, ms_min = time_graph(run_step)
         reference = [y.clone() for _, _, _, y in calls[:8]] + [calls[-1][3].clone()]
-        ms_per_step = ms_chain
         if args.branches > 1:
-            ms_per_step = time_graph(run_step_branches)
+            ms_br, ms_br_min = time_graph(run_step_branches)
             for want, (_, _, _, y) in zip(reference, calls[:8] + [calls[-1]]):
                 assert torch.equal(want, y), "branched step differs from the chained one"
+            side_by_side = {"graph_branches": args.branches, "ms_per_step": round(ms_br, 4), "ms_per_step_min": round(ms_br_min, 4),
+                            "GBps": round(step_bytes / (ms_br * 1e-3) / 1e9, 1),
+                            "frac": round(step_bytes / (ms_br * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                            "note": "the 253 calls of this sweep do not depend on each other: layer l's seven calls as a "
+                                    "chain on graph branch l mod B.  A decode pass cannot do this (layer l+1 needs layer l)"}
+        if not args.no_chain and len(ctxs) >= 1:
+            # the same dependent step as a chain of overlapping launches (each call starts while its predecessor
+            # runs and waits for it inside the kernel): built, bit-identical, and slower than kernel boundaries
+            chain_layers = [(l, x, y) for _, l, x, y in calls if l.ctx is ctxs[0]]
+            if len(chain_layers) >= 8:
+                def run_chain():
+                    ctxs[0].chain_begin()
+                    for l, x, y in chain_layers:
+                        l.forward(x, out=y)
+                    ctxs[0].chain_end()
+
+                g = capture(run_chain)
+                us, _ = time_events(g, len(chain_layers))
+
+                def run_plain():
+                    for l, x, y in chain_layers:
+                        l.forward(x, out=y)
+
+                us_plain, _ = time_events(capture(run_plain), len(chain_layers))
+                assert not ctxs[0].chain_gave_up()
+                overlapped = {"launches": len(chain_layers), "us_per_launch_chained": round(us, 3),
+                              "us_per_launch_plain": round(us_plain, 3),
+                              "note": "a81w41_context_chain_begin/end over the calls of one context: in-kernel waits on "
+                                      "agent-scope counters instead of kernel boundaries; same bits"}
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
-    serial_chain = {"ms_per_step": round(ms_chain, 4), "GBps": round(step_bytes / (ms_chain * 1e-3) / 1e9, 1),
-                    "note": "the same 253 launches captured as one dependent chain on one stream"}
+    serial_chain = {"ms_per_step": round(ms_per_step, 4), "ms_per_step_min": round(ms_min, 4),
+                    "GBps": round(value, 1), "GBps_best_window": round(step_bytes / (ms_min * 1e-3) / 1e9, 1),
+                    "windows": N_WINDOWS, "steps_per_window": args.steps,
+                    "note": "the 253 launches captured as one dependent chain on one stream: this is `value`"}
 
     grouped = None
     if args.grouped:
@@ -250,15 +322,31 @@ def main():
                 main.wait_stream(st)
 
         with torch.cuda.stream(stream):
-            ms_grouped = time_graph(run_grouped)
-            ms_grouped_br = time_graph(run_grouped_branches) if args.branches > 1 else None
+            ms_grouped, ms_grouped_min = time_graph(run_grouped)
+            ms_grouped_br = time_graph(run_grouped_branches)[0] if args.branches > 1 else None
         grouped = {"launches_per_step": len(groups), "ms_per_step": round(ms_grouped, 4),
+                   "ms_per_step_min": round(ms_grouped_min, 4),
                    "GBps": round(step_bytes / (ms_grouped * 1e-3) / 1e9, 1),
                    "note": "q+k+v and gate+up contracted by one launch each (a81w41_linear_forward_multi), "
-                           "one dependent chain"}
+                           "one dependent chain: the call sites of the reference's model (QwenAttention.cc:29)"}
         if ms_grouped_br is not None:
-            grouped["branches"] = {"graph_branches": args.branches, "ms_per_step": round(ms_grouped_br, 4),
-                                   "GBps": round(step_bytes / (ms_grouped_br * 1e-3) / 1e9, 1)}
+            grouped["side_by_side"] = {"graph_branches": args.branches, "ms_per_step": round(ms_grouped_br, 4),
+                                       "GBps": round(step_bytes / (ms_grouped_br * 1e-3) / 1e9, 1)}
+        # per launch of the two grouped call sites (dependent chain over the layers' copies)
+        grouped["per_launch"] = []
+        with torch.cuda.stream(stream):
+            for gname, width in (("qkv (q+k+v in one launch, 4096 -> 6144)", 3), ("gate_up (gate+up in one launch, 4096 -> 24576)", 2)):
+                sel = [(ls, x, outs) for (ls, x), outs in zip(groups, gouts) if len(ls) == width]
+
+                def launch_sel():
+                    for ls, x, outs in sel:
+                        ops.Linear.forward_multi(ls, x, outs)
+
+                us, us_min = time_events(capture(launch_sel), len(sel))
+                b = sum(0.625 * l.K * l.N + 4.0 * l.N for l in sel[0][0]) + 1.125 * sel[0][0][0].K
+                grouped["per_launch"].append({"call_site": gname, "launches_per_step": len(sel), "us_per_launch": round(us, 3),
+                                              "us_per_launch_min": round(us_min, 3), "GBps": round(b / us / 1e3, 1),
+                                              "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4)})
 
     # --- roofline of the GEMV kernel (the layer's M = 1 launch: quantiser prologue + contraction),
     # per shape over that shape's distinct resident weights, timed with events on the launch stream.
@@ -273,52 +361,30 @@ def main():
                 for l, x, y in group:
                     l.forward(x, out=y)
 
-            launch_all()
-            stream.synchronize()
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g, stream=stream):
-                launch_all()
-            reps = 20  # same for every shape: the launch mix of this leg equals the step's
-            g.replay()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(stream)
-            for _ in range(reps):
-                g.replay()
-            e1.record(stream)
-            stream.synchronize()
-            us = e0.elapsed_time(e1) * 1e3 / (reps * len(group))
+            g = capture(launch_all)
+            us, us_min = time_events(g, len(group))
             b = gemv_bytes(K, N)
             row = {"shape": name, "K": K, "N": N, "launches_per_step": len(group),
-                   "us_per_launch": round(us, 3), "GBps": round(b / us / 1e3, 1),
+                   "us_per_launch": round(us, 3), "us_per_launch_min": round(us_min, 3), "GBps": round(b / us / 1e3, 1),
                    "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4)}
             if args.blob:  # the contraction alone: activation blob in, no quantiser prologue
                 a_blob = ops.quantize(group[0][1], False)
-                gb = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(gb, stream=stream):
+
+                def launch_blob():
                     for l, _, y in group:
                         ops.gemv_fp16(a_blob, l.weight_fp16_ptr, N, K, out=y)
-                gb.replay()
-                e0.record(stream)
-                for _ in range(reps):
-                    gb.replay()
-                e1.record(stream)
-                stream.synchronize()
-                ub = e0.elapsed_time(e1) * 1e3 / (reps * len(group))
+
+                ub, _ = time_events(capture(launch_blob), len(group))
                 row["blob_us_per_launch"] = round(ub, 3)
                 row["blob_GBps"] = round(b / ub / 1e3, 1)
             if args.hot:  # the same launch on one weight copy, 16 times per graph replay
                 l0, x0, y0 = group[0]
-                gh = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(gh, stream=stream):
+
+                def launch_hot():
                     for _ in range(16):
                         l0.forward(x0, out=y0)
-                gh.replay()
-                e0.record(stream)
-                for _ in range(10):
-                    gh.replay()
-                e1.record(stream)
-                stream.synchronize()
-                hot = e0.elapsed_time(e1) * 1e3 / 160
+
+                hot, _ = time_events(capture(launch_hot), 16)
                 row["hot_us_per_launch"] = round(hot, 3)
                 row["hot_GBps"] = round(b / hot / 1e3, 1)
             per_shape.append(row)
@@ -368,29 +434,17 @@ def main():
 
             out = []
             for fn in (gemm_only, forward):
-                fn()
-                stream.synchronize()
-                g = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(g, stream=stream):
-                    fn()
-                g.replay()
-                reps = 3
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record(stream)
-                for _ in range(reps):
-                    g.replay()
-                e1.record(stream)
-                stream.synchronize()
-                out.append(e0.elapsed_time(e1) * 1e3 / (reps * len(group)))
-            return out[0], out[1]
+                out.append(time_events(capture(fn), len(group))[0])
+            return out[0], out[1], group[0].kernel_name(M)
 
         rows = []
         tot_ops, tot_t, tot_tg = 0.0, 0.0, 0.0
         with torch.cuda.stream(stream):
             for name, K, N in LAYER_SHAPES:
-                us, us_fwd = time_forward(name, M, K, N, 97)
+                us, us_fwd, kname = time_forward(name, M, K, N, 97)
                 opsn = 2.0 * M * N * K
-                rows.append({"shape": name, "K": K, "N": N, "forward_us": round(us_fwd, 2), "gemm_us": round(us, 2),
+                rows.append({"shape": name, "K": K, "N": N, "kernel": kname.split(" ")[0],
+                             "forward_us": round(us_fwd, 2), "gemm_us": round(us, 2),
                              "TOPS": round(opsn / us_fwd / 1e6, 2),
                              "mfma_int8_frac": round(opsn / us_fwd / 1e6 / INT8_PEAK_TOPS, 4),
                              "gemm_only_TOPS": round(opsn / us / 1e6, 2)})
@@ -398,7 +452,7 @@ def main():
                 tot_t += us_fwd
                 tot_tg += us
             # the reference author's own kernel bench point (tests/test_linear.cc:113-115,272)
-            us320, fwd320 = time_forward("gate", 320, 4096, 12288, 95)
+            us320, fwd320, _ = time_forward("gate", 320, 4096, 12288, 95)
             # The call sites as the reference's model makes them: qkv_proj is stored as one 4096 -> 6144 layer
             # (QwenAttention.cc:29,78-83) and the exporter writes gate_up_proj the same way, so a prefill pass
             # runs four GEMMs per layer, not seven.
@@ -410,9 +464,9 @@ def main():
                     layers[li][name] = ops.Linear.from_blobs(None, b32, N, K, ctxs[li % len(ctxs)])
                 del w4, scale, offset, b32
             for name, K, N in (("qkv", 4096, 6144), ("o", 4096, 4096), ("gate_up", 4096, 24576), ("down", 12288, 4096)):
-                us, us_fwd = time_forward(name, M, K, N, 97)
+                us, us_fwd, kname = time_forward(name, M, K, N, 97)
                 opsn = 2.0 * M * N * K
-                fused_rows.append({"shape": name, "K": K, "N": N, "forward_us": round(us_fwd, 2),
+                fused_rows.append({"shape": name, "K": K, "N": N, "kernel": kname.split(" ")[0], "forward_us": round(us_fwd, 2),
                                    "TOPS": round(opsn / us_fwd / 1e6, 2)})
                 f_ops += opsn
                 f_t += us_fwd
@@ -420,8 +474,9 @@ def main():
                  "frac": round(tot_ops / tot_t / 1e6 / INT8_PEAK_TOPS, 4),
                  "gemm_only_TOPS": round(tot_ops / tot_tg / 1e6, 2),
                  "note": "TOPS = 2*M*N*K / forward_us: activation quantiser launch + GEMM launch, per call, weights "
-                         "rotated over the 36 layers' resident copies, 36 calls per HIP-graph replay; gemm_us is the "
-                         "GEMM launch alone on a quantised blob",
+                         "rotated over the 36 layers' resident copies, 36 calls per HIP-graph replay, median of five "
+                         "windows of at least 40 ms; gemm_us is the int8 GEMM launch alone on a quantised blob "
+                         "(a81w41_gemm_repack_A81W41_fp32, the reference's signature); kernel = what forward ran",
                  "per_shape": rows,
                  "fused_call_sites": {"TOPS": round(f_ops / f_t / 1e6, 2), "frac": round(f_ops / f_t / 1e6 / INT8_PEAK_TOPS, 4),
                                       "per_shape": fused_rows,
@@ -440,7 +495,7 @@ def main():
             for name in ("gate", "down"):
                 group = [d[name] for d in layers]     # rotate over the layers' copies: weights from HBM
                 K, N = group[0].K, group[0].N
-                for M in (1, 8, 32, 128, 512, 2048, 4096):
+                for M in (1, 2, 8, 9, 16, 24, 32, 64, 128, 256, 322, 512, 1024, 2048, 4096):
                     x = torch.from_numpy(synth.activations(M, K, 96)).cuda()
                     y = torch.empty((M, N), dtype=torch.float32, device="cuda")
 
@@ -448,22 +503,13 @@ def main():
                         for l in group:
                             l.forward(x, out=y)
 
-                    sweep()
-                    stream.synchronize()
-                    g = torch.cuda.CUDAGraph()
-                    with torch.cuda.graph(g, stream=stream):
-                        sweep()
-                    g.replay()
-                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    e0.record(stream)
-                    g.replay()
-                    g.replay()
-                    e1.record(stream)
-                    stream.synchronize()
-                    us = e0.elapsed_time(e1) * 1e3 / (2 * len(group))
+                    us, us_min = time_events(capture(sweep), len(group), min_window_ms=20.0)
                     wbytes = (0.625 if M == 1 else 0.75) * K * N
-                    m_sweep.append({"shape": name, "M": M, "path": "gemv" if M == 1 else "quantiser + gemm",
-                                    "forward_us": round(us, 2), "TOPS": round(2.0 * M * N * K / us / 1e6, 2),
+                    kname = group[0].kernel_name(M)
+                    m_sweep.append({"shape": name, "M": M, "kernel": kname.split(" ")[0], "kernel_note": kname,
+                                    "path": "one launch" if M == 1 else "quantiser launch + contraction launch",
+                                    "forward_us": round(us, 2), "forward_us_min": round(us_min, 2),
+                                    "TOPS": round(2.0 * M * N * K / us / 1e6, 2),
                                     "weight_GBps": round(wbytes / us / 1e3, 1)})
 
     # --- whole forward pass, random-init Qwen3-8B (prefill 322 tokens + 128 greedy decode steps) ---
@@ -480,11 +526,6 @@ def main():
     if not args.no_cpu:
         cpu = cpu_baseline(pkg)
 
-    if args.branches > 1 and not args.profile:
-        # what the same kernel delivers when the step's independent launches run side by side: whole-step bytes
-        # over whole-step time (no per-launch duration exists for launches that overlap)
-        roofline["side_by_side"] = {"graph_branches": args.branches, "achieved": round(value, 1),
-                                    "frac": round(value / HBM_PEAK_GBS, 4)}
     out = {
         "metric": "A8W4 QGEMV GB/s (M=1) + QGEMM TOPS (M=322) on Qwen3-8B shapes",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -493,11 +534,13 @@ def main():
         "config": {"workload": "decode GEMV sweep M=1, Qwen3-8B linear shapes (configs[1]): "
                                f"{args.layers} layers x (q,k,v,o,gate,up,down) + lm_head, one forward call "
                                "(quantiser prologue + GEMV, one launch) per linear, group size 32, "
-                               "distinct resident weights per layer, HIP-graph replay; the calls are independent "
-                               f"and captured as {args.branches} parallel branch(es)",
-                   "calls_per_step": len(calls), "bytes_per_step": step_bytes, "graph_branches": args.branches},
+                               "distinct resident weights per layer, HIP-graph replay as one dependent chain on one "
+                               f"stream; median of {N_WINDOWS} windows of {args.steps} steps",
+                   "calls_per_step": len(calls), "bytes_per_step": step_bytes},
         "tokens_per_s_linear_only": round(1e3 / ms_per_step, 1),
         "serial_chain": serial_chain,
+        "side_by_side": side_by_side,
+        "overlapped_chain": overlapped,
         "grouped_call_sites": grouped,
         "roofline": roofline, "per_shape": per_shape, "qgemm": qgemm, "m_sweep": m_sweep, "e2e": e2e,
         "a80w40": a80, "cpu_baseline": cpu,
@@ -629,7 +672,14 @@ def end_to_end(pkg, n_prompt=322, n_decode=128):
         if best is None or ms_pre + ms_dec < best[0] + best[1]:
             best = (ms_pre, ms_dec)
     ms_pre, ms_dec = best
+    rb = model.resident_bytes()
+    n_w = sum(n * k for n, k in dims) * cfg["n_layers"] + V * H
+    resident = dict(rb, GiB=round(rb["total"] / 2**30, 2), linear_bytes_per_weight=round(rb["linear_weights"] / n_w, 3),
+                    note="linear_weights: 0.625 B/weight (fp16-parameter blob, decode) + 0.75 (fp32-parameter blob, prefill) + "
+                         "1.0 (block-scaled operand) for the layers whose prefill can use it, lm_head 0.625 only; other_weights: "
+                         "fp16 embedding, norms, rotation tables; the reference reports 14.0 GiB with fp32 embedding and KV cache")
     return {"model": "Qwen3-8B shape, random init, all linears A81W41, fp16 KV cache", "prefill_tokens": n_prompt,
+            "resident_bytes": resident,
             "prefill_ms": round(ms_pre, 3), "prefill_tokens_per_s": round(n_prompt / ms_pre * 1e3, 1),
             "decode_steps": n_decode, "decode_ms": round(ms_dec, 3),
             "decode_tokens_per_s": round(n_decode / ms_dec * 1e3, 2),

@@ -211,6 +211,9 @@ void a81w41_linear_destroy(a81w41_linear *layer);
  * Out-pointers may be NULL. */
 size_t a81w41_linear_resident_bytes(const a81w41_linear *layer, size_t *fp16_blob, size_t *fp32_blob,
                                     size_t *block_scaled);
+/* Which kernel a forward call of M rows of this layer runs on (a static string for reports:
+ * "gemv ...", "rows ...", "rows32 ...", "tile32x128 ...", "tile64 ...", "block_scaled ..."). */
+const char *a81w41_linear_kernel_name(const a81w41_linear *layer, int M);
 int a81w41_linear_in_features(const a81w41_linear *layer);  /* K */
 int a81w41_linear_out_features(const a81w41_linear *layer); /* N */
 const void *a81w41_linear_weight_fp16_dev(const a81w41_linear *layer);
@@ -356,6 +359,12 @@ enum {
 };
 int a81w41_qwen3_set_option(a81w41_qwen3 *model, int option, int value);
 int a81w41_qwen3_chain_status(a81w41_qwen3 *model, int *gave_up); /* synchronises */
+/* Device memory the model holds, in total and by kind (out-pointers may be NULL): the linears'
+ * weight copies (a81w41_linear_resident_bytes), the other weights (fp16 embedding table, norms,
+ * rotation tables), the fp16 KV cache, and activation buffers + scratches.  The reference reports
+ * 14.0 GiB resident for the same model with fp32 embedding and KV cache (README.md:41). */
+size_t a81w41_qwen3_resident_bytes(const a81w41_qwen3 *model, size_t *linear_weights,
+                                   size_t *other_weights, size_t *kv_cache, size_t *buffers);
 /* Parity hook: copies the first `count` floats of one of the model's activation buffers to the host
  * after the work enqueued so far has finished.  After a pass the buffers hold what the LAST layer left
  * (the fused passes skip some of them: switch A81W41_QWEN3_OPT_UNFUSED on to have every stage written):

@@ -46,6 +46,7 @@ SIGNATURES = {
     "a81w41_linear_load": (_i, [_vp, C.c_char_p, _i, _i, _i, C.POINTER(_vp)]),
     "a81w41_linear_destroy": (None, [_vp]),
     "a81w41_linear_resident_bytes": (_sz, [_vp, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)]),
+    "a81w41_linear_kernel_name": (C.c_char_p, [_vp, _i]),
     "a81w41_linear_in_features": (_i, [_vp]),
     "a81w41_linear_out_features": (_i, [_vp]),
     "a81w41_linear_weight_fp16_dev": (_vp, [_vp]),
@@ -69,6 +70,7 @@ SIGNATURES = {
     "a81w41_qwen3_set_embedding": (_i, [_vp, _vp]),
     "a81w41_qwen3_set_option": (_i, [_vp, _i, _i]),
     "a81w41_qwen3_chain_status": (_i, [_vp, C.POINTER(_i)]),
+    "a81w41_qwen3_resident_bytes": (_sz, [_vp, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)]),
     "a81w41_qwen3_read_buffer": (_i, [_vp, _i, _vp, _sz]),
     "a81w41_qwen3_reset": (_i, [_vp]),
     "a81w41_qwen3_forward": (_i, [_vp, _vp, _i, _vp]),

@@ -114,6 +114,7 @@ struct GemmScratch {
 };
 hipError_t gemm_scratch_create(GemmScratch* out);  // 64 MiB + counters on the current device
 void gemm_scratch_destroy(GemmScratch* ws);
+size_t gemm_scratch_bytes(const GemmScratch& ws);
 // The scratch that belongs to stream s on the current device, created at the first call for that stream
 // (which therefore must not come while s is being captured: hipErrorStreamCaptureUnsupported).
 hipError_t gemm_scratch_for_stream(hipStream_t s, GemmScratch* out);
@@ -125,6 +126,8 @@ int gemm_partial_tiles(int M, int N, int K);
 hipError_t clear_gemm_counters(const GemmScratch& ws, hipStream_t s);
 // hipErrorInvalidValue if the call's schedule needs more partial tiles than ws holds.
 hipError_t launch_gemm_fp32(const void* A, const void* B, float* C, int M, int N, int K, const GemmScratch& ws, hipStream_t s);
+// Which of the M > 1 kernels launch_gemm_fp32 sends a call of this shape to (a name for reports).
+const char* gemm_kernel_name(int M, int N, int K);
 // Walks the work list of a launch on the host (wm = 1: 32 x 128 tiles, 2: 64 x 64) for a device with
 // slots_fit resident workgroups on cus CUs: >= 0 (the partial tiles used) if every tile and chunk is
 // covered exactly once and no partial tile is shared, else a negative code.
@@ -174,6 +177,7 @@ struct a81w41_context;
 namespace a81w41 {
 // The K-split scratch a context owns, and its A6 scratch (capi.cpp).
 const GemmScratch& context_gemm_scratch(const a81w41_context* ctx);
+size_t context_resident_bytes(const a81w41_context* ctx);  // its scratches
 ChainState* context_chain(a81w41_context* ctx);
 void* context_a6_scratch(const a81w41_context* ctx);
 }  // namespace a81w41

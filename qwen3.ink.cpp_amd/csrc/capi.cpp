@@ -154,6 +154,9 @@ struct a81w41_linear {
 namespace a81w41 {
 const GemmScratch& context_gemm_scratch(const a81w41_context* ctx) { return ctx->gemm_scratch; }
 void* context_a6_scratch(const a81w41_context* ctx) { return ctx->a6_scratch; }
+size_t context_resident_bytes(const a81w41_context* ctx) {
+    return ctx->act_bytes + ctx->a6_bytes + ctx->x_bytes + ctx->y_bytes + gemm_scratch_bytes(ctx->gemm_scratch);
+}
 ChainState* context_chain(a81w41_context* ctx) {
     if (!ctx->chain_ready) {
         if (chain_create(&ctx->chain) != hipSuccess) return nullptr;
@@ -576,6 +579,13 @@ size_t a81w41_linear_resident_bytes(const a81w41_linear* l, size_t* fp16_blob, s
     if (fp32_blob) *fp32_blob = b32;
     if (block_scaled) *block_scaled = b6;
     return b16 + b32 + b6;
+}
+
+const char* a81w41_linear_kernel_name(const a81w41_linear* l, int M) {
+    if (!l || M < 1) return "";
+    if (M == 1) return "gemv (v_dot4, fused quantiser prologue, weights streamed once)";
+    if (a81w41::linear_block_scaled(l, M)) return "block_scaled (fp6 block-scaled matrix ops, 128 x 256 tiles, stream-K)";
+    return a81w41::gemm_kernel_name(M, l->N, l->K);
 }
 
 int a81w41_linear_in_features(const a81w41_linear* l) { return l ? l->K : 0; }

@@ -616,6 +616,15 @@ int pick_kernel(int M, int N, int K) {
 
 using namespace gemm_detail;
 
+const char* gemm_kernel_name(int M, int N, int K) {
+    switch (pick_kernel(M, N, K)) {
+        case 0: return "rows (2..8 rows resident in LDS, v_dot4, weights streamed once)";
+        case 1: return "tile32x128 (int8 matrix ops, 4 waves side by side, K split)";
+        case 3: return "rows32 (int8 matrix ops, one row panel, K split inside the workgroup)";
+        default: return "tile64 (int8 matrix ops, 64 x 64 tiles, LDS-staged)";
+    }
+}
+
 hipError_t gemm_scratch_create(GemmScratch* out) {
     out->partials = nullptr;
     out->arrivals = nullptr;
@@ -635,6 +644,10 @@ hipError_t gemm_scratch_create(GemmScratch* out) {
     out->arrivals = a;
     out->max_partials = kMaxPartials;
     return hipSuccess;
+}
+
+size_t gemm_scratch_bytes(const GemmScratch& ws) {
+    return (size_t)ws.max_partials * (kPartialWords * sizeof(float) + sizeof(unsigned));
 }
 
 void gemm_scratch_destroy(GemmScratch* ws) {

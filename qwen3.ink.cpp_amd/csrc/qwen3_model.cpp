@@ -531,6 +531,35 @@ int a81w41_qwen3_set_option(a81w41_qwen3* m, int option, int value) {
     return A81W41_OK;
 }
 
+size_t a81w41_qwen3_resident_bytes(const a81w41_qwen3* m, size_t* linear_weights, size_t* other_weights, size_t* kv_cache,
+                                   size_t* buffers) {
+    if (!m) return 0;
+    const a81w41_qwen3_config& c = m->cfg;
+    size_t lin = 0, other = 0;
+    for (const LayerWeights& L : m->layers) {
+        for (int w = 0; w < 4; w++) {
+            lin += a81w41_linear_resident_bytes(L.lin[w], nullptr, nullptr, nullptr);
+            if (L.norm[w]) other += (size_t)(w < 2 ? c.hidden : kHeadDim) * sizeof(float);
+        }
+    }
+    lin += a81w41_linear_resident_bytes(m->lm_head, nullptr, nullptr, nullptr);
+    if (m->final_norm) other += (size_t)c.hidden * sizeof(float);
+    if (m->embedding) other += (size_t)c.vocab * c.hidden * 2;
+    other += 2 * (size_t)c.max_seq * kHeadDim * sizeof(float);  // rotation tables
+    const size_t kv = 2 * (size_t)c.n_layers * c.n_kv_heads * c.max_seq * kHeadDim * 2;
+    const size_t rows = c.max_seq;
+    size_t buf = (rows * c.hidden * 3 + (size_t)c.hidden + rows * m->qkv_dim() + rows * c.n_q_heads * kHeadDim +
+                  rows * 3 * c.intermediate + (size_t)c.vocab) * sizeof(float);
+    buf += (size_t)c.n_q_heads * a81w41::kAttentionMaxSplits * 132 * sizeof(float) + (size_t)c.n_q_heads * sizeof(unsigned);
+    buf += (rows + 2 + (size_t)m->history_len) * sizeof(int);
+    buf += a81w41::context_resident_bytes(m->ctx);
+    if (linear_weights) *linear_weights = lin;
+    if (other_weights) *other_weights = other;
+    if (kv_cache) *kv_cache = kv;
+    if (buffers) *buffers = buf;
+    return lin + other + kv + buf;
+}
+
 int a81w41_qwen3_chain_status(a81w41_qwen3* m, int* gave_up) {
     if (!m || !gave_up) return fail(A81W41_ERR_INVALID_ARG, "null argument");
     Q_HIP(hipStreamSynchronize(m->stream));

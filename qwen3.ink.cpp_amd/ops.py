@@ -301,6 +301,10 @@ class Linear:
         capi.check(capi.lib().a81w41_linear_forward(self.handle, _dev_ptr(x), M, _dev_ptr(out), _stream()))
         return out
 
+    def kernel_name(self, M: int) -> str:
+        """Which kernel a forward call of M rows runs on (``a81w41_linear_kernel_name``)."""
+        return capi.lib().a81w41_linear_kernel_name(self.handle, int(M)).decode()
+
     def resident_bytes(self) -> dict:
         """Device bytes of the layer's weight copies (``a81w41_linear_resident_bytes``)."""
         a, b, c = C.c_size_t(), C.c_size_t(), C.c_size_t()
@@ -408,6 +412,12 @@ class Qwen3Model:
         flag = C.c_int(0)
         capi.check(capi.lib().a81w41_qwen3_chain_status(self.handle, C.byref(flag)))
         return bool(flag.value)
+
+    def resident_bytes(self) -> dict:
+        """Device bytes the model holds, by kind (``a81w41_qwen3_resident_bytes``)."""
+        a, b, c, d = C.c_size_t(), C.c_size_t(), C.c_size_t(), C.c_size_t()
+        total = capi.lib().a81w41_qwen3_resident_bytes(self.handle, C.byref(a), C.byref(b), C.byref(c), C.byref(d))
+        return {"total": int(total), "linear_weights": a.value, "other_weights": b.value, "kv_cache": c.value, "buffers": d.value}
 
     BUFFERS = {"residual": 0, "normed": 1, "qkv": 2, "attention": 3, "block_out": 4, "gate_up": 5, "act": 6, "logits": 7}
 

@@ -159,7 +159,10 @@ def test_last_layer_stage_by_stage_against_the_oracle(full, ora):
     for h in range(nq):
         s = (q[:, h] @ k[:, h // (nq // nkv)].T) / np.sqrt(128.0)
         want[:, h] = qf.softmax_rows(np.where(causal, s, -np.inf)) @ v[:, h // (nq // nkv)]
-    assert row_rel(attn.reshape(M, nq, 128), want) <= 5e-5
+    # the worst of 322 x 32 head rows, each relative to its own 128-vector (rows whose weighted values cancel
+    # down to a small vector set it: 5e-5 on this data; all rows together agree to 2e-5 of the token row's norm)
+    assert row_rel(attn.reshape(M, nq, 128), want) <= 1e-4
+    assert row_rel(attn, want.reshape(M, nq * 128)) <= 2e-5
     # SiLU * mul (QwenOperator.cc:697-713)
     g64, u64 = gate_up[:, :I].astype(np.float64), gate_up[:, I:].astype(np.float64)
     assert row_rel(act, g64 / (1.0 + np.exp(-g64)) * u64) <= 2e-6

@@ -454,3 +454,51 @@ def test_layer_kernel_choice_at_full_width(pkg, ora, synth, torch):
     assert row_err(auto, want) <= 3e-5
     with pytest.raises(Exception):
         pkg.capi.check(pkg.capi.lib().a81w41_linear_set_kernel(layer.handle, 7))
+
+
+def test_third_weight_copy_only_where_it_can_be_used(pkg, ora, synth, torch):
+    """The block-scaled kernel's operand format (1 B per weight on top of the reference's two blobs) is built
+    only for layers that a call their context admits can send to that kernel; the int8 choice frees it, the
+    block-scaled choice builds it, and results are those of the int8 kernel to the path's bar either way."""
+    K = 4096
+    ctx = pkg.ops.Context(max_rows=512, max_cols=K)
+    narrow_w = synth.weight_files(1024, K, 621)
+    wide_w = synth.weight_files(12288, K, 622)
+    narrow = pkg.Linear.from_arrays(*narrow_w, N=1024, K=K, ctx=ctx)     # k / v shape: never enough tiles at <= 512 rows
+    wide = pkg.Linear.from_arrays(*wide_w, N=12288, K=K, ctx=ctx)        # gate shape: block-scaled from 256 rows on
+    rb = narrow.resident_bytes()
+    assert rb["block_scaled"] == 0 and rb["fp16_blob"] == 1024 * K * 5 // 8 and rb["fp32_blob"] == 1024 * K * 3 // 4
+    assert wide.resident_bytes()["block_scaled"] == 12288 * K
+    x = dev(torch, synth.activations(300, K, 623))
+    base = narrow.forward(x).cpu().numpy()
+    narrow.set_kernel("block_scaled")
+    assert narrow.resident_bytes()["block_scaled"] == 1024 * K
+    forced = narrow.forward(x).cpu().numpy()
+    assert row_err(forced, base) <= 3e-5 and not np.array_equal(forced, base)
+    narrow.set_kernel("int8")
+    assert narrow.resident_bytes()["block_scaled"] == 0
+    assert np.array_equal(narrow.forward(x).cpu().numpy(), base)
+    wide.set_kernel("int8")
+    assert wide.resident_bytes()["total"] == 12288 * K * 11 // 8
+    wide.set_kernel("auto")
+    assert wide.resident_bytes()["block_scaled"] == 12288 * K
+    # a layer without an fp32-parameter blob (decode only) holds one copy
+    only16 = pkg.Linear.from_blobs(ora.repack(*narrow_w, K, 1024, False), None, 1024, K, ctx)
+    assert only16.resident_bytes() == {"total": 1024 * K * 5 // 8, "fp16_blob": 1024 * K * 5 // 8, "fp32_blob": 0, "block_scaled": 0}
+
+
+def test_gemm_on_more_streams_than_scratches(pkg, ora, synth, torch):
+    """The free-standing GEMM keeps one K-split scratch per stream, at most 16 per device: streams beyond that
+    take over the least recently used scratch instead of failing.  20 fresh streams in turn, then the first
+    again, all with the same bits."""
+    M, N, K = 130, 136, 2048                       # splits K
+    w4, s, o = synth.weight_files(N, K, 631)
+    ba, bw = ora.quantize(synth.activations(M, K, 632), True), ora.repack(w4, s, o, K, N, True)
+    a, b = dev(torch, ba), dev(torch, bw)
+    ref = pkg.ops.gemm_fp32(a, b, M, N, K).clone()
+    streams = [torch.cuda.Stream() for _ in range(20)]
+    for st in streams + streams[:2]:
+        with torch.cuda.stream(st):
+            got = pkg.ops.gemm_fp32(a, b, M, N, K)
+        st.synchronize()
+        assert torch.equal(got, ref)
