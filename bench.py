@@ -507,7 +507,8 @@ def main():
                     wbytes = (0.625 if M == 1 else 0.75) * K * N
                     kname = group[0].kernel_name(M)
                     m_sweep.append({"shape": name, "M": M, "kernel": kname.split(" ")[0], "kernel_note": kname,
-                                    "path": "one launch" if M == 1 else "quantiser launch + contraction launch",
+                                    "path": "one launch (quantiser fused in the prologue)" if kname.split(" ")[0] in ("gemv", "rows_fused")
+                                            else "quantiser launch + contraction launch",
                                     "forward_us": round(us, 2), "forward_us_min": round(us_min, 2),
                                     "TOPS": round(2.0 * M * N * K / us / 1e6, 2),
                                     "weight_GBps": round(wbytes / us / 1e3, 1)})

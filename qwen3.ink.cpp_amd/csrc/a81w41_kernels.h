@@ -154,6 +154,10 @@ int gemm_fp6_plan_selfcheck(int M, int N, int K, int slots);
 // launch_gemm_fp32 when gemm_rows_fits(): same arguments and results within the same tolerance.
 bool gemm_rows_fits(int M, int K);
 hipError_t launch_gemm_rows_fp32(const void* A, const void* B, float* C, int M, int N, int K, hipStream_t s);
+// The same with the fp32-parameter quantiser fused in front (x: M x K fp32, 16-byte aligned; a_out, may be null,
+// receives the M*K/64 blocks of 80 B): one launch for quantiser + contraction, where that is the faster form.
+bool gemm_rows_fused_preferred(int M, int K);
+hipError_t launch_gemm_rows_fused(const float* x, void* a_out, const void* B, float* C, int M, int N, int K, hipStream_t s);
 // 9 <= M <= 32: one row panel, operands loaded straight into registers, K cut inside and between workgroups.
 int gemm_rows32_split(int N, int K);
 hipError_t launch_gemm_rows32_fp32(const void* A, const void* B, float* C, int M, int N, int K, const GemmScratch& ws,

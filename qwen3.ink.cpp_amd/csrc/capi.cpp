@@ -584,6 +584,7 @@ size_t a81w41_linear_resident_bytes(const a81w41_linear* l, size_t* fp16_blob, s
 const char* a81w41_linear_kernel_name(const a81w41_linear* l, int M) {
     if (!l || M < 1) return "";
     if (M == 1) return "gemv (v_dot4, fused quantiser prologue, weights streamed once)";
+    if (a81w41::gemm_rows_fused_preferred(M, l->K)) return "rows_fused (2..8 rows quantised in the prologue, resident in LDS, v_dot4, one launch)";
     if (a81w41::linear_block_scaled(l, M)) return "block_scaled (fp6 block-scaled matrix ops, 128 x 256 tiles, stream-K)";
     return a81w41::gemm_kernel_name(M, l->N, l->K);
 }
@@ -697,6 +698,13 @@ int a81w41_linear_forward(a81w41_linear* l, const float* x_dev, int M, float* y_
             HIP_TRY(a81w41::launch_quantize_a6(x_dev, ctx->act_scratch, ctx->a6_scratch, M, l->K, static_cast<hipStream_t>(stream)));
             HIP_TRY(a81w41::launch_gemm_fp6(ctx->a6_scratch, l->w6, y_dev, M, l->N, l->K, ctx->gemm_scratch,
                                             static_cast<hipStream_t>(stream)));
+            return A81W41_OK;
+        }
+        if ((reinterpret_cast<uintptr_t>(x_dev) & 15) == 0 && a81w41::gemm_rows_fused_preferred(M, l->K)) {
+            // few rows: one launch, every workgroup quantises the rows itself, workgroup 0 also fills the scratch
+            if (int st = contract_args_ok(x_dev, l->w32, y_dev, M, l->N, l->K)) return st;
+            HIP_TRY(a81w41::launch_gemm_rows_fused(x_dev, ctx->act_scratch, l->w32, y_dev, M, l->N, l->K,
+                                                   static_cast<hipStream_t>(stream)));
             return A81W41_OK;
         }
         if (int st = a81w41_quantize_row_q8_1_repack_fp32(x_dev, ctx->act_scratch, (int64_t)M * l->K, stream)) return st;

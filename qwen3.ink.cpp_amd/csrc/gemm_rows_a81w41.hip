@@ -12,6 +12,12 @@
 //   acc = fma(float(idot), fl(dA*dW), acc);  acc = fma(mW, sA, acc)
 // (quantized_gemx_kernels.cc:509-512).  Partial sums are reduced across lanes, then across the
 // waves of the column group in a fixed order (deterministic output).
+//
+// FUSED: the rows come as fp32 and every workgroup quantises them itself on its way into LDS
+// (quantize_row_q8_1_repack_fp32, quantized_gemx_kernels.cc:803-911, the same device function as the
+// stand-alone quantiser; workgroup 0 also writes the 80 B blocks out, so the caller's scratch holds what
+// the reference's buffer would).  One launch instead of two; every workgroup reads M*K*4 bytes of rows, so it
+// pays for few rows only (gemm_rows_fused_preferred).
 #include "a81w41_kernels.h"
 #include "quantize_common.h"
 
@@ -55,11 +61,12 @@ __device__ __forceinline__ void lds_barrier() {
     __builtin_amdgcn_sched_barrier(0);
 }
 
-template <int MR>
+template <int MR, bool FUSED>
 __global__ __launch_bounds__(64 * kRowsWaves) void gemm_rows_a81w41_fp32_kernel(const uint8_t* __restrict__ A,
                                                                               const uint8_t* __restrict__ B,
                                                                               float* __restrict__ C, int M, int N,
-                                                                              int nb_n, int nb_k, int wpg_log2) {
+                                                                              int nb_n, int nb_k, int wpg_log2,
+                                                                              uint8_t* __restrict__ a_out) {
     extern __shared__ __align__(16) uint32_t lds[];  // MR*nb_k*24 words of activations, then 2*kRowsWaves*32*MR floats
     constexpr int kThreads = 64 * kRowsWaves;
     const int tid = threadIdx.x;
@@ -80,7 +87,50 @@ __global__ __launch_bounds__(64 * kRowsWaves) void gemm_rows_a81w41_fp32_kernel(
     // Activation rows -> LDS images (rows past M are zero: they contribute nothing and are not stored).
     // Loads are requested four per thread at a time, and the first weight blocks right behind the first
     // four: the vector-memory counter retires in order, so whatever is requested first is waited for first.
-    {
+    auto request_first_weights = [&]() {
+        __builtin_amdgcn_sched_barrier(0);
+        const int blk = wig * kBlocksPerStep + blk_in_step;
+        rows_load(cur, B + ((size_t)g * nb_k + blk) * kWBlock32, sub, g < nb_n && blk < nb_k);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    if (FUSED) {
+        // one float4 per thread and slice, eight lanes per 32-block; row m's blocks follow row m-1's
+        const float4* x4 = reinterpret_cast<const float4*>(A);
+        const int n_vec = M * nb_k * 16, n_all = MR * nb_k * 16;
+        constexpr int kChunk = 4;
+        for (int base = 0; base < n_all; base += kChunk * kThreads) {
+            float4 v[kChunk];
+#pragma unroll
+            for (int u = 0; u < kChunk; u++) {
+                const int i = base + u * kThreads + tid;
+                v[u] = (i < n_vec) ? x4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+            if (base == 0) request_first_weights();
+#pragma unroll
+            for (int u = 0; u < kChunk; u++) {
+                if (base + u * kThreads >= n_all) break;  // empty slice (uniform over the workgroup)
+                const int i = base + u * kThreads + tid;
+                const Quant4 qz = quantize_float4_of_block32(v[u]);  // rows past M: zeros in, zero block out
+                if (i < n_all) {
+                    const int b32 = i >> 3, p = i & 7, b = b32 >> 1, lh = b32 & 1;  // b = row*nb_k + sb
+                    uint32_t* dst = lds + b * kLdsWordsPerSb;
+                    dst[lds_q_word(lh, p)] = qz.packed;
+                    if (p == 0) {
+                        dst[12 * lh + 8] = __float_as_uint(qz.d);
+                        dst[12 * lh + 9] = __float_as_uint(qz.ssum);
+                    }
+                    if (a_out != nullptr && blockIdx.x == 0 && i < n_vec) {
+                        uint8_t* ob = a_out + (size_t)b * kABlock32;
+                        *reinterpret_cast<uint32_t*>(ob + 16 + 32 * lh + 4 * p) = qz.packed;
+                        if (p == 0) {
+                            reinterpret_cast<float*>(ob)[lh] = qz.d;
+                            reinterpret_cast<float*>(ob)[2 + lh] = qz.ssum;
+                        }
+                    }
+                }
+            }
+        }
+    } else {
         const uint4* A128 = reinterpret_cast<const uint4*>(A);  // five 16-byte pieces per 80 B block
         const int n_pieces = M * nb_k * 5, n_all = MR * nb_k * 5;
         constexpr int kChunk = 4;
@@ -91,12 +141,7 @@ __global__ __launch_bounds__(64 * kRowsWaves) void gemm_rows_a81w41_fp32_kernel(
                 const int i = base + u * kThreads + tid;
                 v[u] = (i < n_pieces) ? A128[i] : make_uint4(0, 0, 0, 0);
             }
-            if (base == 0) {
-                __builtin_amdgcn_sched_barrier(0);
-                const int blk = wig * kBlocksPerStep + blk_in_step;
-                rows_load(cur, B + ((size_t)g * nb_k + blk) * kWBlock32, sub, g < nb_n && blk < nb_k);
-                __builtin_amdgcn_sched_barrier(0);
-            }
+            if (base == 0) request_first_weights();
 #pragma unroll
             for (int u = 0; u < kChunk; u++) {
                 const int i = base + u * kThreads + tid;
@@ -231,11 +276,11 @@ size_t rows_lds_bytes(int K) {
     return ((size_t)MR * (K / 64) * kLdsWordsPerSb + 2 * kRowsWaves * 32 * MR) * sizeof(uint32_t);
 }
 
-template <int MR>
-hipError_t launch_rows(const void* A, const void* B, float* C, int M, int N, int K, hipStream_t s) {
+template <int MR, bool FUSED>
+hipError_t launch_rows(const void* A, const void* B, float* C, int M, int N, int K, void* a_out, hipStream_t s) {
     const size_t lds = rows_lds_bytes<MR>(K);
     if (lds > 64 * 1024) {  // a kernel gets 64 KiB of dynamic LDS without asking (asked per call: per device, no shared flag)
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_rows_a81w41_fp32_kernel<MR>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_rows_a81w41_fp32_kernel<MR, FUSED>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimitBytes);
         if (e != hipSuccess) return e;
     }
@@ -247,9 +292,25 @@ hipError_t launch_rows(const void* A, const void* B, float* C, int M, int N, int
     const int wgs = (nb_n + slots - 1) / slots;
     const int max_grid = lds * 2 <= (size_t)kLdsLimitBytes ? 512 : 256;  // what the CUs hold at once
     const int grid = wgs < max_grid ? wgs : max_grid;
-    hipLaunchKernelGGL((gemm_rows_a81w41_fp32_kernel<MR>), dim3(grid), dim3(64 * kRowsWaves), lds, s,
-                       static_cast<const uint8_t*>(A), static_cast<const uint8_t*>(B), C, M, N, nb_n, nb_k, wpg_log2);
+    hipLaunchKernelGGL((gemm_rows_a81w41_fp32_kernel<MR, FUSED>), dim3(grid), dim3(64 * kRowsWaves), lds, s,
+                       static_cast<const uint8_t*>(A), static_cast<const uint8_t*>(B), C, M, N, nb_n, nb_k, wpg_log2,
+                       static_cast<uint8_t*>(a_out));
     return hipGetLastError();
+}
+
+template <bool FUSED>
+hipError_t launch_rows_any(const void* A, const void* B, float* C, int M, int N, int K, void* a_out, hipStream_t s) {
+    switch (M) {
+        case 1: return launch_rows<1, FUSED>(A, B, C, M, N, K, a_out, s);
+        case 2: return launch_rows<2, FUSED>(A, B, C, M, N, K, a_out, s);
+        case 3: return launch_rows<3, FUSED>(A, B, C, M, N, K, a_out, s);
+        case 4: return launch_rows<4, FUSED>(A, B, C, M, N, K, a_out, s);
+        case 5: return launch_rows<5, FUSED>(A, B, C, M, N, K, a_out, s);
+        case 6: return launch_rows<6, FUSED>(A, B, C, M, N, K, a_out, s);
+        case 7: return launch_rows<7, FUSED>(A, B, C, M, N, K, a_out, s);
+        case 8: return launch_rows<8, FUSED>(A, B, C, M, N, K, a_out, s);
+        default: return hipErrorInvalidValue;
+    }
 }
 
 }  // namespace
@@ -263,17 +324,23 @@ bool gemm_rows_fits(int M, int K) {
 }
 
 hipError_t launch_gemm_rows_fp32(const void* A, const void* B, float* C, int M, int N, int K, hipStream_t s) {
-    switch (M) {
-        case 1: return launch_rows<1>(A, B, C, M, N, K, s);
-        case 2: return launch_rows<2>(A, B, C, M, N, K, s);
-        case 3: return launch_rows<3>(A, B, C, M, N, K, s);
-        case 4: return launch_rows<4>(A, B, C, M, N, K, s);
-        case 5: return launch_rows<5>(A, B, C, M, N, K, s);
-        case 6: return launch_rows<6>(A, B, C, M, N, K, s);
-        case 7: return launch_rows<7>(A, B, C, M, N, K, s);
-        case 8: return launch_rows<8>(A, B, C, M, N, K, s);
-        default: return hipErrorInvalidValue;
-    }
+    return launch_rows_any<false>(A, B, C, M, N, K, nullptr, s);
+}
+
+// Whether the one-launch form (rows quantised by every workgroup) beats quantiser launch + contraction launch.
+// Every workgroup reads and quantises all M*K values.  Measured on MI355X (one launch against two, us per call):
+// K = 4096, N = 12288: 2 rows 10.9 / 12.2, 3 rows 12.7 / 12.8, 4 rows 14.5 / 13.4, 8 rows 22.5 / 18.4;
+// N = 4096: 6.4 / 7.4, 7.6 / 7.8, 8.5 / 8.0; N = 1024: 5.2 / 6.2, 6.5 / 6.7, 7.4 / 7.1; K = 12288: 2 rows 16.9 / 13.0.
+bool gemm_rows_fused_preferred(int M, int K) {
+    const int mode = tuning_env_int("A81W41_ROWS_FUSED");  // tuning builds: 1 = never, 2 = whenever it fits
+    if (mode == 1) return false;
+    if (!gemm_rows_fits(M, K)) return false;
+    if (mode == 2) return true;
+    return (long long)M * K <= 12288;
+}
+
+hipError_t launch_gemm_rows_fused(const float* x, void* a_out, const void* B, float* C, int M, int N, int K, hipStream_t s) {
+    return launch_rows_any<true>(x, B, C, M, N, K, a_out, s);
 }
 
 }  // namespace a81w41

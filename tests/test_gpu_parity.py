@@ -502,3 +502,28 @@ def test_gemm_on_more_streams_than_scratches(pkg, ora, synth, torch):
             got = pkg.ops.gemm_fp32(a, b, M, N, K)
         st.synchronize()
         assert torch.equal(got, ref)
+
+
+@pytest.mark.parametrize("M,N,K", [(2, 8, 64), (2, 12288, 4096), (3, 1024, 4096), (2, 4096, 6144), (6, 136, 1088), (8, 40, 1536),
+                                   (4, 64, 3072), (3, 4096, 4160)])
+def test_few_row_forward_quantises_in_its_prologue(pkg, ora, synth, torch, M, N, K):
+    """Calls with few rows and M*K <= 12288 are one launch: every workgroup quantises the fp32 rows itself
+    (quantize_row_q8_1_repack_fp32's arithmetic) on their way into LDS, workgroup 0 also writes the 80 B blocks
+    to the scratch.  Scratch bit-exact, output the same bits as the contraction of the oracle-quantised rows by
+    the same kernel without the prologue, all within the bar; shapes just above the limit take two launches."""
+    w4, s, o = synth.weight_files(N, K, 641)
+    s = s * np.float32(1.0371)
+    x = synth.activations(M, K, 642, outliers=True)
+    x[M - 1, :64] = 0.0                             # an all-zero block: d = 0, id = 0
+    ctx = pkg.ops.Context(max_rows=8, max_cols=K)
+    bw = ora.repack(w4, s, o, K, N, True)
+    layer = pkg.Linear.from_blobs(None, bw, N, K, ctx)
+    fused = M * K <= 12288
+    assert layer.kernel_name(M).startswith("rows_fused" if fused else "rows ")
+    got = layer.forward(dev(torch, x))
+    ba = ora.quantize(x, True)
+    assert np.array_equal(ctx.activation_scratch(M * K // 64 * 80).cpu().numpy(), ba)
+    want = ora.gemm_fp32(ba, bw, M, N, K)
+    assert row_err(got.cpu().numpy(), want) <= 5e-6
+    # the same kernel without the prologue, on the quantised rows (the free-standing entry point)
+    assert torch.equal(got, pkg.ops.gemm_fp32(dev(torch, ba), dev(torch, bw), M, N, K))
