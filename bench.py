@@ -220,14 +220,16 @@ def main():
 
     def time_events(graph, units_per_replay, min_window_ms=40.0):
         """A captured graph timed with events on the launch stream: N_WINDOWS windows of at least min_window_ms
-        each.  -> (median, minimum) microseconds per unit."""
+        each (with --profile: of exactly --steps replays each, so that every leg's graph is replayed equally often
+        and a kernel's average duration in a trace of the run is an average over the step's own launch mix).
+        -> (median, minimum) microseconds per unit."""
         graph.replay()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(stream)
         graph.replay()
         e1.record(stream)
         stream.synchronize()
-        reps = max(2, int(min_window_ms / max(e0.elapsed_time(e1), 1e-3)) + 1)
+        reps = args.steps if args.profile else max(2, int(min_window_ms / max(e0.elapsed_time(e1), 1e-3)) + 1)
         out = []
         for _ in range(N_WINDOWS):
             e0.record(stream)
