@@ -43,7 +43,7 @@ HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 # this script (FETCH_SIZE, WRITE_SIZE), each scaled by the same counter's reading for a 256 MiB
 # copy kernel (factors 2.000 and 1.000); summary in profiles/gemv_decode_sweep_hbm_traffic.md.
 # Only valid for the default 36-layer workload; reported as null otherwise.
-MEASURED_GEMV_TRAFFIC_BYTES_PER_LAUNCH = 19009269
+MEASURED_GEMV_TRAFFIC_BYTES_PER_LAUNCH = 19006282
 TRAFFIC_SOURCE = ("profiles/gemv_decode_sweep_hbm_traffic.md: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of "
                   "`bench.py --profile` (not measured in this run)")
 INT8_PEAK_TOPS = 5000.0    # MI355X dense int8 matrix peak
