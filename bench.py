@@ -624,10 +624,11 @@ def a80w40_leg(pkg, M):
             "note": "gemv: bytes-weighted over 36 x seven shapes + lm_head; gemm time includes the operand rewrite"}
 
 
-def end_to_end(pkg, n_prompt=322, n_decode=128):
+def build_e2e_model(pkg, n_prompt=322):
     """Random-init Qwen3-8B (36 layers, hidden 4096, 32 q / 8 kv heads x 128, intermediate 12288,
     vocab 151936, RoPE theta 1e6, fp16 KV cache), every linear A81W41 from the seeded generator
-    (one weight set per shape, a distinct HBM copy per layer); uniform random prompt ids."""
+    (one weight set per shape, a distinct HBM copy per layer); uniform random prompt ids.
+    -> (model, prompt, number of linear weights)"""
     ops, synth = pkg.ops, pkg.synth
     cfg = dict(n_layers=N_LAYERS, hidden=4096, n_q_heads=32, n_kv_heads=8, intermediate=12288, vocab=151936, max_seq=512)
     t0 = time.time()
@@ -665,6 +666,12 @@ def end_to_end(pkg, n_prompt=322, n_decode=128):
     del emb
     print(f"[bench] Qwen3-8B random-init model resident after {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
     prompt = rng.integers(0, V, size=n_prompt).astype(np.int32)
+    n_w = sum(n * k for n, k in dims) * cfg["n_layers"] + V * H
+    return model, prompt, n_w
+
+
+def time_generation(model, prompt, n_decode):
+    """Best of 3 identical greedy generations -> (tokens, prefill ms, decode ms)."""
     best = None
     for rep in range(3):   # first repetition warms caches and code objects
         model.reset()
@@ -674,9 +681,13 @@ def end_to_end(pkg, n_prompt=322, n_decode=128):
         assert np.array_equal(toks, first), "greedy generation is not repeatable"
         if best is None or ms_pre + ms_dec < best[0] + best[1]:
             best = (ms_pre, ms_dec)
-    ms_pre, ms_dec = best
+    return toks, best[0], best[1]
+
+
+def end_to_end(pkg, n_prompt=322, n_decode=128):
+    model, prompt, n_w = build_e2e_model(pkg, n_prompt)
+    toks, ms_pre, ms_dec = time_generation(model, prompt, n_decode)
     rb = model.resident_bytes()
-    n_w = sum(n * k for n, k in dims) * cfg["n_layers"] + V * H
     resident = dict(rb, GiB=round(rb["total"] / 2**30, 2), linear_bytes_per_weight=round(rb["linear_weights"] / n_w, 3),
                     note="linear_weights: 0.625 B/weight (fp16-parameter blob, decode) + 0.75 (fp32-parameter blob, prefill) + "
                          "1.0 (block-scaled operand) for the layers whose prefill can use it, lm_head 0.625 only; other_weights: "
