@@ -113,13 +113,13 @@ int a81w41_gemm_repack_A81W41_fp32(const void *A_repack_dev, const void *B_repac
 int a81w41_gemm_repack_A81W41_fp32_static(const void *A_repack_dev, const void *B_repack_dev,
                                           float *C_dev, int M, int N, int K, void *stream);
 
-/* Test hook, host only (no device is touched): walks the work list the M > 8 kernels would be
- * launched with for an M x N x K call on a device that holds `resident_workgroups` of them on
- * `cus` compute units (tile = 2: 64 x 64 tiles, 1: 32 x 128 tiles).  Returns the number of
+/* Test hook, host only (no device is touched): walks the work list the 64 x 64-tile kernel would be
+ * launched with for an M x N x K call on a device that holds `resident_workgroups` of its workgroups on
+ * `cus` compute units.  Returns the number of
  * partial tiles the K split parks (>= 0) if every tile and every K chunk is covered exactly
  * once, the tile numbering is one-to-one and no two chunks share a partial tile; a negative
  * code names the violated property. */
-int a81w41_gemm_schedule_selfcheck(int M, int N, int K, int resident_workgroups, int cus, int tile);
+int a81w41_gemm_schedule_selfcheck(int M, int N, int K, int resident_workgroups, int cus);
 
 /* Test hook, host only: the same for the layer object's M > 32 kernel (128 x 128 tiles, the (tile,
  * 32-block) units of a launch cut into equal contiguous runs): every unit exactly once, contributor
@@ -212,7 +212,7 @@ void a81w41_linear_destroy(a81w41_linear *layer);
 size_t a81w41_linear_resident_bytes(const a81w41_linear *layer, size_t *fp16_blob, size_t *fp32_blob,
                                     size_t *block_scaled);
 /* Which kernel a forward call of M rows of this layer runs on (a static string for reports:
- * "gemv ...", "rows ...", "rows32 ...", "tile32x128 ...", "tile64 ...", "block_scaled ..."). */
+ * "gemv ...", "rows ...", "rows_fused ...", "rows32 ...", "rows32_staged ...", "tile64 ...", "block_scaled ..."). */
 const char *a81w41_linear_kernel_name(const a81w41_linear *layer, int M);
 int a81w41_linear_in_features(const a81w41_linear *layer);  /* K */
 int a81w41_linear_out_features(const a81w41_linear *layer); /* N */

@@ -28,7 +28,7 @@ SIGNATURES = {
     "a81w41_gemv_repack_A81W41_fp16": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "a81w41_gemm_repack_A81W41_fp32": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "a81w41_gemm_repack_A81W41_fp32_static": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
-    "a81w41_gemm_schedule_selfcheck": (_i, [_i, _i, _i, _i, _i, _i]),
+    "a81w41_gemm_schedule_selfcheck": (_i, [_i, _i, _i, _i, _i]),
     "a81w41_gemm_fp6_plan_selfcheck": (_i, [_i, _i, _i, _i]),
     "a81w41_block_idot": (_i, [_vp, _i, _vp, _i, _vp, _i, _i, _i, _vp]),
     "a81w41_repack_w80_weight": (_i, [_i, _i, _i, _vp, _vp, _vp]),

@@ -31,7 +31,10 @@ constexpr int kABlock32 = 80;   // q8_repack_1x2_fp32
 
 // write_sums = false: the scaled-sum fields of the blocks are left as they are
 // (quantize_row_q8_0_repack, quantized_gemx_kernels.cc:584-682).
-hipError_t launch_quantize(const float* x, void* y, int64_t nb64, bool fp32, hipStream_t s, bool write_sums = true);
+// y_by_superblock (fp32 parameters, at most 32 rows of nb_k super-blocks; may be null): a second copy of the blocks,
+// block (row, sb) at (32 sb + row) * 80, for launch_gemm_rows32_fp32's staged form.
+hipError_t launch_quantize(const float* x, void* y, int64_t nb64, bool fp32, hipStream_t s, bool write_sums = true,
+                           void* y_by_superblock = nullptr, int nb_k = 0);
 // Persistent GEMV grid: at most this many workgroups (8 per CU on 256 CUs).
 constexpr int kGemvMaxGrid = 2048;
 constexpr int kLdsLimitBytes = 160 * 1024;
@@ -128,10 +131,10 @@ hipError_t clear_gemm_counters(const GemmScratch& ws, hipStream_t s);
 hipError_t launch_gemm_fp32(const void* A, const void* B, float* C, int M, int N, int K, const GemmScratch& ws, hipStream_t s);
 // Which of the M > 1 kernels launch_gemm_fp32 sends a call of this shape to (a name for reports).
 const char* gemm_kernel_name(int M, int N, int K);
-// Walks the work list of a launch on the host (wm = 1: 32 x 128 tiles, 2: 64 x 64) for a device with
+// Walks the work list of a launch of the 64 x 64-tile kernel on the host for a device with
 // slots_fit resident workgroups on cus CUs: >= 0 (the partial tiles used) if every tile and chunk is
 // covered exactly once and no partial tile is shared, else a negative code.
-int gemm_schedule_selfcheck(int M, int N, int K, int slots_fit, int cus, int wm);
+int gemm_schedule_selfcheck(int M, int N, int K, int slots_fit, int cus);
 // ---- the layer object's M > 32 path: block-scaled fp6 matrix ops on private operand formats (gemm_fp6_a81w41.hip)
 // A6: quantised activations as two 4-bit pieces per value in fp6 patterns, W6: weight codes as fp6 patterns,
 // both with fp32 parameters, in 32-row / 32-column panels.  Rows and columns are padded to multiples of 32.
@@ -159,9 +162,13 @@ hipError_t launch_gemm_rows_fp32(const void* A, const void* B, float* C, int M, 
 bool gemm_rows_fused_preferred(int M, int K);
 hipError_t launch_gemm_rows_fused(const float* x, void* a_out, const void* B, float* C, int M, int N, int K, hipStream_t s);
 // 9 <= M <= 32: one row panel, operands loaded straight into registers, K cut inside and between workgroups.
-int gemm_rows32_split(int N, int K);
+int gemm_rows32_split(int N, int K, bool staged = false);
+// staged: operands through wave-private LDS stages (wide layers); a_by_superblock (staged only, may be null): the copy of
+// A that launch_quantize writes with a super-block's rows next to each other (32 row slots per super-block).
 hipError_t launch_gemm_rows32_fp32(const void* A, const void* B, float* C, int M, int N, int K, const GemmScratch& ws,
-                                   hipStream_t s);
+                                   hipStream_t s, bool staged = false, const void* a_by_superblock = nullptr);
+bool gemm_rows32_staged_preferred(int M, int N, int K);  // whether launch_gemm_fp32 would take the staged form
+size_t gemm_rows32_a_by_superblock_bytes(int K);
 // w80: codes count as code - 8 (the A80W40 variant).
 hipError_t launch_block_idot(const void* A, bool a_fp32, const void* B, bool b_fp32, int32_t* out,
                              int M, int N, int K, hipStream_t s, bool w80 = false);

@@ -368,10 +368,10 @@ int a81w41_gemm_repack_A81W41_fp32_static(const void* A_repack_dev, const void* 
     return A81W41_OK;
 }
 
-int a81w41_gemm_schedule_selfcheck(int M, int N, int K, int resident_workgroups, int cus, int tile) {
-    if (M < 1 || !shape_ok(N, K) || cus < 1 || resident_workgroups < cus || resident_workgroups % cus || (tile != 1 && tile != 2))
+int a81w41_gemm_schedule_selfcheck(int M, int N, int K, int resident_workgroups, int cus) {
+    if (M < 1 || !shape_ok(N, K) || cus < 1 || resident_workgroups < cus || resident_workgroups % cus)
         return fail(A81W41_ERR_INVALID_ARG, "bad arguments") * -100;
-    return a81w41::gemm_schedule_selfcheck(M, N, K, resident_workgroups, cus, tile);
+    return a81w41::gemm_schedule_selfcheck(M, N, K, resident_workgroups, cus);
 }
 
 int a81w41_gemm_fp6_plan_selfcheck(int M, int N, int K, int resident_workgroups) {
@@ -705,6 +705,19 @@ int a81w41_linear_forward(a81w41_linear* l, const float* x_dev, int M, float* y_
             if (int st = contract_args_ok(x_dev, l->w32, y_dev, M, l->N, l->K)) return st;
             HIP_TRY(a81w41::launch_gemm_rows_fused(x_dev, ctx->act_scratch, l->w32, y_dev, M, l->N, l->K,
                                                    static_cast<hipStream_t>(stream)));
+            return A81W41_OK;
+        }
+        if (a81w41::gemm_rows32_staged_preferred(M, l->N, l->K) &&
+            a81w41::gemm_rows32_a_by_superblock_bytes(l->K) <= ctx->a6_bytes) {
+            // up to 32 rows on a wide layer: the quantiser also writes the blocks with a super-block's rows next to each
+            // other (into the scratch of the block-scaled kernel's operands, which such a call does not use), and the
+            // contraction stages its activations from there; same arithmetic, same bits as from the 80 B blocks alone
+            if (int st = contract_args_ok(ctx->act_scratch, l->w32, y_dev, M, l->N, l->K)) return st;
+            if (reinterpret_cast<uintptr_t>(x_dev) & 3) return fail(A81W41_ERR_INVALID_ARG, "x must be 4-byte aligned");
+            HIP_TRY(a81w41::launch_quantize(x_dev, ctx->act_scratch, (int64_t)M * l->K / 64, true, static_cast<hipStream_t>(stream),
+                                            true, ctx->a6_scratch, l->K / 64));
+            HIP_TRY(a81w41::launch_gemm_rows32_fp32(ctx->act_scratch, l->w32, y_dev, M, l->N, l->K, ctx->gemm_scratch,
+                                                    static_cast<hipStream_t>(stream), true, ctx->a6_scratch));
             return A81W41_OK;
         }
         if (int st = a81w41_quantize_row_q8_1_repack_fp32(x_dev, ctx->act_scratch, (int64_t)M * l->K, stream)) return st;

@@ -20,8 +20,9 @@
 // what it waits for -- LDS, matrix results, the barrier, copies -- the other three waves of its SIMD
 // fill.  (Software pipelines over two sets of product registers, which limit a CU to two workgroups,
 // were 6-15 % slower; so was operand lookahead at three per CU.)  The K range of the tiles of the
-// last, partial round of the grid may be split (see Schedule).  Calls with few rows use the same
-// kernel with idle waves, or 32 x 128 tiles (template argument WM).
+// last, partial round of the grid may be split (see Schedule).  Calls with at most 32 rows go to the
+// kernels made for them (gemm_rows_a81w41.hip, gemm_rows32_a81w41.hip); this one serves them only as the
+// free-standing fallback of shapes those do not take.
 //
 // Staging.  Per super-block a workgroup needs
 //   A stage: its rows' whole 80 B blocks, row stride 80 B (conflict-free 128-bit reads)
@@ -71,22 +72,16 @@ __device__ __forceinline__ void copy_wave_16B_to_lds(const uint8_t* global_src, 
 }
 
 constexpr int kTileThreads = 256;
-constexpr int kPartialWords = 4096;  // one fp32 partial tile (64 x 64 or 32 x 128)
+constexpr int kPartialWords = 4096;  // one fp32 partial tile (64 x 64)
 
-// Two arrangements of the four waves of a workgroup (template argument WM = waves along M):
-//   WM = 2: 2 x 2 waves, 64 x 64 tile.  A stage is 320 A chunks + 192 B chunks of 16 B, two full
-//           64-lane copies per wave.
-//   WM = 1: 1 x 4 waves, 32 x 128 tile, for calls with at most 32 rows (no wave idles on rows that
-//           do not exist).  A stage is 160 A chunks + 384 B chunks; every wave makes three copies:
-//           8 rows (40 lanes) and twice two weight blocks (48 lanes).
-template <int WM>
+// The four waves of a workgroup are 2 x 2 over a 64 x 64 tile.  A stage is 320 activation chunks + 192 weight
+// chunks of 16 bytes: two full 64-lane copies per wave.
 struct Geom {
-    static constexpr int kTileM = 32 * WM, kTileN = 128 / WM;
+    static constexpr int kTileM = 64, kTileN = 64;
     static constexpr int kStageB = kTileM * kABlock32;                    // offset of the B part
-    static constexpr int kStage = kStageB + (kTileN / 8) * kWBlock32;     // 8192 or 8704 bytes
-    static constexpr int kCopies = WM == 2 ? 2 : 3;                       // per wave and stage
-    // Stages in LDS; all but one are in flight.  Deeper rings were measured for both arrangements
-    // (6 and 8 stages): no gain for the 64 x 64 tiles, 10-40 % slower for the 32 x 128 ones.
+    static constexpr int kStage = kStageB + (kTileN / 8) * kWBlock32;     // 8192 bytes
+    static constexpr int kCopies = 2;                                     // per wave and stage
+    // Stages in LDS; all but one are in flight.  Deeper rings (6 and 8 stages) were measured: no gain.
     static constexpr int kRing = 4;
     static constexpr int kLdsBytes = kRing * kStage;
 };
@@ -117,34 +112,25 @@ struct TileRead {     // per-lane LDS byte offsets inside a stage
 // slot 24*gl + (k + 2*(gl%4)) % 24.  The 32 lanes of a half wave read the same chunk index of
 // four consecutive blocks; the rotation spreads those over all 32 LDS banks (unrotated, the
 // four blocks would hit the same eight).
-template <int WM>
 __device__ __forceinline__ uint32_t b_slot_byte(int gl, int k, int jj) {
-    return Geom<WM>::kStageB + (24 * gl + (k + 2 * (gl & 3)) % 24) * 16 + 4 * (jj & 3);
+    return Geom::kStageB + (24 * gl + (k + 2 * (gl & 3)) % 24) * 16 + 4 * (jj & 3);
 }
 
-// This wave's direct-to-LDS copies of a stage for super-block sb: two full ones (WM = 2), or one of
-// 40 lanes and two of 48 (WM = 1; a copy moves lanes 0..n-1 only, its LDS target stays contiguous).
-template <int WM>
+// This wave's two direct-to-LDS copies of a stage for super-block sb.
 __device__ __forceinline__ void tile_issue(const TileDma& d, uint8_t* lds, int buf, int sb, int lane) {
 #pragma unroll
-    for (int i = 0; i < Geom<WM>::kCopies; i++) {
+    for (int i = 0; i < Geom::kCopies; i++) {
         // keep the wave-uniform part of the address in scalar registers: saddr + 32-bit lane offset
         const uint64_t ub = reinterpret_cast<uint64_t>(d.base[i]) + (uint64_t)sb * d.step[i];
         const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)ub);
         const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(ub >> 32));
         const uint8_t* sbase = reinterpret_cast<const uint8_t*>(((uint64_t)hi << 32) | lo);
-        uint8_t* dst = lds + buf * Geom<WM>::kStage + d.lds_off[i];
-        if (WM == 2) {
-            copy_wave_16B_to_lds(sbase + d.voff[i], dst);
-        } else {
-            if (lane < (i == 0 ? 40 : 48)) copy_wave_16B_to_lds(sbase + d.voff[i], dst);
-        }
+        copy_wave_16B_to_lds(sbase + d.voff[i], lds + buf * Geom::kStage + d.lds_off[i]);
     }
 }
 
-template <int WM>
 __device__ __forceinline__ void tile_read(TileOps& o, const uint8_t* lds, int buf, const TileRead& rd, int kh) {
-    const uint8_t* st = lds + buf * Geom<WM>::kStage;
+    const uint8_t* st = lds + buf * Geom::kStage;
     const uint8_t* row = st + rd.a;
     o.Al = *reinterpret_cast<const v4i*>(row + 16 + 16 * kh);
     o.Ah = *reinterpret_cast<const v4i*>(row + 48 + 16 * kh);
@@ -226,33 +212,32 @@ __host__ __device__ __forceinline__ void tile_xy(int tau, int tiles_m, int tiles
 #define A81W41_TILE_READY(BUF, SB)                                                  \
     do {                                                                            \
         __builtin_amdgcn_sched_barrier(0); /* nothing above may sink below */      \
-        wait_vmcnt<(kRing - 2) * Geom<WM>::kCopies>();                              \
+        wait_vmcnt<(kRing - 2) * Geom::kCopies>();                                  \
         __builtin_amdgcn_s_barrier();                                               \
         __builtin_amdgcn_sched_barrier(0); /* no LDS read below may rise above */  \
-        tile_issue<WM>(dma, lds, (BUF), k0 + min((SB), n_sb - 1), lane);            \
+        tile_issue(dma, lds, (BUF), k0 + min((SB), n_sb - 1), lane);                \
     } while (0)
 
-template <int WM>
 __device__ __forceinline__ void tile_kernel_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                  float* __restrict__ C, int M, int N, int nb_k, const Schedule& sc,
                                                  float* __restrict__ partials, unsigned* __restrict__ arrivals, uint8_t* lds,
                                                  unsigned& s_arrived) {
-    constexpr int kTileM = Geom<WM>::kTileM, kTileN = Geom<WM>::kTileN, kRing = Geom<WM>::kRing;
+    constexpr int kTileM = Geom::kTileM, kTileN = Geom::kTileN, kRing = Geom::kRing;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 31, kh = lane >> 5;
     const int nb_n = N >> 3;
-    const int row0 = WM == 2 ? (wave >> 1) * 32 : 0, col0 = WM == 2 ? (wave & 1) * 32 : wave * 32;
+    const int row0 = (wave >> 1) * 32, col0 = (wave & 1) * 32;
 
     TileRead rd;
     {
         rd.a = (row0 + r) * kABlock32;
         const int col = col0 + r, gl = col >> 3, jj = col & 7;
-        rd.dW = b_slot_byte<WM>(gl, 2 * kh + (jj >> 2), jj);
-        rd.mW = b_slot_byte<WM>(gl, 4 + 2 * kh + (jj >> 2), jj);
+        rd.dW = b_slot_byte(gl, 2 * kh + (jj >> 2), jj);
+        rd.mW = b_slot_byte(gl, 4 + 2 * kh + (jj >> 2), jj);
 #pragma unroll
-        for (int t = 0; t < 4; t++) rd.w[t] = b_slot_byte<WM>(gl, 8 + 2 * (4 * kh + t) + (jj >> 2), jj);
+        for (int t = 0; t < 4; t++) rd.w[t] = b_slot_byte(gl, 8 + 2 * (4 * kh + t) + (jj >> 2), jj);
     }
 
     for (int item = blockIdx.x; item < sc.items; item += gridDim.x) {
@@ -273,51 +258,29 @@ __device__ __forceinline__ void tile_kernel_body(const uint8_t* __restrict__ A, 
         tile_xy(tau, sc.tiles_m, sc.tiles_n, sc.band, tx, ty);
         const int m_base = ty * kTileM, n_base = tx * kTileN;
 
-        // WM = 2: copy q = i*4 + wave of a stage moves chunks 64q..64q+63: copies 0..4 are activation rows
-        // (5 chunks per row), 5..7 weight blocks.  WM = 1: wave w copies rows 8w..8w+7 (lane = 5*row + piece)
-        // and, twice, weight blocks 4w+2j, 4w+2j+1 (lane = 24*block + slot).  Rows past M alias the last
-        // row and column groups past N the last group; neither is ever stored.
+        // Copy q = i*4 + wave of a stage moves chunks 64q..64q+63: copies 0..4 are activation rows (5 chunks per
+        // row), 5..7 weight blocks.  Rows past M alias the last row and column groups past N the last group;
+        // neither is ever stored.
         TileDma dma;
-        if (WM == 2) {
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                const int q = i * 4 + wave;
-                const int c = q * 64 + lane;
-                dma.lds_off[i] = q * 1024;
-                if (q < 5) {
-                    const int row = c / 5, piece = c - row * 5;
-                    const int m_rel = min(m_base + row, M - 1) - m_base;
-                    dma.base[i] = A + (size_t)m_base * nb_k * kABlock32;
-                    dma.step[i] = kABlock32;
-                    dma.voff[i] = (uint32_t)m_rel * nb_k * kABlock32 + 16 * piece;
-                } else {
-                    const int s = c - 320;
-                    const int gl = s / 24, pos = s - gl * 24;
-                    const int k = (pos - 2 * (gl & 3) + 24) % 24;  // slot pos of block gl holds chunk k
-                    const int g_rel = min((n_base >> 3) + gl, nb_n - 1) - (n_base >> 3);
-                    dma.base[i] = B + (size_t)(n_base >> 3) * nb_k * kWBlock32;
-                    dma.step[i] = kWBlock32;
-                    dma.voff[i] = (uint32_t)g_rel * nb_k * kWBlock32 + 16 * k;
-                }
-            }
-        } else {
-            {
-                const int l = min(lane, 39), row = 8 * wave + l / 5, piece = l % 5;
+        for (int i = 0; i < 2; i++) {
+            const int q = i * 4 + wave;
+            const int c = q * 64 + lane;
+            dma.lds_off[i] = q * 1024;
+            if (q < 5) {
+                const int row = c / 5, piece = c - row * 5;
                 const int m_rel = min(m_base + row, M - 1) - m_base;
-                dma.base[0] = A + (size_t)m_base * nb_k * kABlock32;
-                dma.step[0] = kABlock32;
-                dma.voff[0] = (uint32_t)m_rel * nb_k * kABlock32 + 16 * piece;
-                dma.lds_off[0] = wave * 8 * kABlock32;
-            }
-#pragma unroll
-            for (int j = 0; j < 2; j++) {
-                const int l = min(lane, 47), gl = 4 * wave + 2 * j + l / 24, pos = l % 24;
+                dma.base[i] = A + (size_t)m_base * nb_k * kABlock32;
+                dma.step[i] = kABlock32;
+                dma.voff[i] = (uint32_t)m_rel * nb_k * kABlock32 + 16 * piece;
+            } else {
+                const int s = c - 320;
+                const int gl = s / 24, pos = s - gl * 24;
                 const int k = (pos - 2 * (gl & 3) + 24) % 24;  // slot pos of block gl holds chunk k
                 const int g_rel = min((n_base >> 3) + gl, nb_n - 1) - (n_base >> 3);
-                dma.base[1 + j] = B + (size_t)(n_base >> 3) * nb_k * kWBlock32;
-                dma.step[1 + j] = kWBlock32;
-                dma.voff[1 + j] = (uint32_t)g_rel * nb_k * kWBlock32 + 16 * k;
-                dma.lds_off[1 + j] = Geom<WM>::kStageB + (4 * wave + 2 * j) * kWBlock32;
+                dma.base[i] = B + (size_t)(n_base >> 3) * nb_k * kWBlock32;
+                dma.step[i] = kWBlock32;
+                dma.voff[i] = (uint32_t)g_rel * nb_k * kWBlock32 + 16 * k;
             }
         }
 
@@ -332,7 +295,7 @@ __device__ __forceinline__ void tile_kernel_body(const uint8_t* __restrict__ A, 
         // workgroups fit a CU; what a wave waits for (LDS, matrix results, the barrier, copies) the
         // other three waves of its SIMD fill.
 #pragma unroll
-        for (int st = 0; st < kRing - 1; st++) tile_issue<WM>(dma, lds, st, k0 + min(st, n_sb - 1), lane);
+        for (int st = 0; st < kRing - 1; st++) tile_issue(dma, lds, st, k0 + min(st, n_sb - 1), lane);
         if (wave_live) {
             for (int t = 0; t < n_sb; t += kRing) {
 #pragma unroll
@@ -342,7 +305,7 @@ __device__ __forceinline__ void tile_kernel_body(const uint8_t* __restrict__ A, 
                     if (u < n_sb) {
                         TileOps o;
                         TileProd F;
-                        tile_read<WM>(o, lds, p, rd, kh);
+                        tile_read(o, lds, p, rd, kh);
                         tile_mfma(o, F, acc);
                         tile_epilogue(F, acc);
                     }
@@ -427,16 +390,7 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
     extern __shared__ __align__(16) uint8_t lds[];  // kRing stages
     __shared__ unsigned s_arrived;
     const Schedule sc = {tiles_m, tiles_n, whole, r, c, chunk, whole + r * c, band};
-    tile_kernel_body<2>(A, B, C, M, N, nb_k, sc, partials, arrivals, lds, s_arrived);
-}
-
-__global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void gemm_a81w41_tile32x128_kernel(
-    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, int M, int N, int nb_k, int tiles_m, int tiles_n, int whole,
-    int r, int c, int chunk, int band, float* __restrict__ C, float* __restrict__ partials, unsigned* __restrict__ arrivals) {
-    extern __shared__ __align__(16) uint8_t lds[];  // kRing stages
-    __shared__ unsigned s_arrived;
-    const Schedule sc = {tiles_m, tiles_n, whole, r, c, chunk, whole + r * c, band};
-    tile_kernel_body<1>(A, B, C, M, N, nb_k, sc, partials, arrivals, lds, s_arrived);
+    tile_kernel_body(A, B, C, M, N, nb_k, sc, partials, arrivals, lds, s_arrived);
 }
 
 // ---- scratch of the K-split path --------------------------------------------------------------
@@ -481,15 +435,10 @@ hipError_t device_info_locked(DeviceInfo*& out) {
     if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
     DeviceInfo& d = g_dev[dev];
     if (d.slots == 0) {
-        int per_cu = 0, per_cu_small = 0, cus = 0;
+        int per_cu = 0, cus = 0;
         e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(&gemm_a81w41_tile64_kernel),
-                                                         kTileThreads, Geom<2>::kLdsBytes);
+                                                         kTileThreads, Geom::kLdsBytes);
         if (e != hipSuccess) return e;
-        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_small,
-                                                         reinterpret_cast<const void*>(&gemm_a81w41_tile32x128_kernel),
-                                                         kTileThreads, Geom<1>::kLdsBytes);
-        if (e != hipSuccess) return e;
-        if (per_cu_small < per_cu) per_cu = per_cu_small;  // one figure for both arrangements
         e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
         if (e != hipSuccess) return e;
         if (per_cu < 1 || cus < 1) return hipErrorInvalidValue;
@@ -507,11 +456,10 @@ __global__ void clear_counters_kernel(unsigned* p, int n) {
 
 // The schedule of one launch (see Schedule): a pure function of the shape and of the device's size.
 // Returns false when the K split the shape calls for needs more than max_partials partial tiles.
-template <int WM>
 bool make_schedule(int M, int N, int K, int slots_fit, int cus, int max_partials, Schedule& sc, int& grid) {
     const int nb_k = K / 64;
-    sc.tiles_m = (M + Geom<WM>::kTileM - 1) / Geom<WM>::kTileM;
-    sc.tiles_n = (N + Geom<WM>::kTileN - 1) / Geom<WM>::kTileN;
+    sc.tiles_m = (M + Geom::kTileM - 1) / Geom::kTileM;
+    sc.tiles_n = (N + Geom::kTileN - 1) / Geom::kTileN;
     const int T = sc.tiles_m * sc.tiles_n;
     // The kernels fit four workgroups per CU; how many the schedule counts on depends on the number of
     // tiles T per CU (measured at N = 4096, M = 128..1536): up to 2 per CU, four (finer K split over
@@ -530,20 +478,13 @@ bool make_schedule(int M, int N, int K, int slots_fit, int cus, int max_partials
     // Split the last, partial round: in two, so that the chunks go to the first (faster) half
     // of the grid; in four when even then less than 3/4 of the grid would have one.
     int c = 1;
-    auto valid = [&](int cc) { return cc >= 1 && cc <= 16 && nb_k % (Geom<WM>::kRing * cc) == 0 && (long long)sc.r * cc <= kMaxPartials; };
+    auto valid = [&](int cc) { return cc >= 1 && cc <= 16 && nb_k % (Geom::kRing * cc) == 0 && (long long)sc.r * cc <= kMaxPartials; };
     if (sc.r > 0) {
         if (valid(2)) c = 2;
         if (valid(4) && sc.r * 4 <= slots * 3 / 4) c = 4;
         // a launch that does not fill the chip once, over a long K: quarters still leave 48 steps per chunk
         // (down_proj at 322 rows: 75.6 against 79.8 us)
         if (valid(4) && sc.whole == 0 && nb_k / 4 >= 48) c = 4;
-        if (WM == 1 && sc.whole == 0) {
-            // Few rows and fewer tiles than the chip has room for: such a call is bound by streaming the
-            // weights once, so cut K as finely as still leaves 8 super-blocks per chunk and one chunk
-            // per workgroup slot.
-            for (int cc : {6, 8, 12, 16})
-                if (valid(cc) && nb_k / cc >= 8 && sc.r * cc <= slots) c = cc;
-        }
         const int env_c = tuning_env_int("A81W41_GEMM_SPLIT");
         if (env_c > 0 && valid(env_c)) c = env_c;
     }
@@ -563,8 +504,6 @@ bool make_schedule(int M, int N, int K, int slots_fit, int cus, int max_partials
     return sc.r * c <= max_partials;
 }
 
-// WM = 2: 64 x 64 tiles; WM = 1: 32 x 128 tiles (calls with at most 32 rows).
-template <int WM>
 hipError_t launch_tiles(const void* A, const void* B, float* C, int M, int N, int K, const GemmScratch& ws, hipStream_t s) {
     DeviceInfo* d = nullptr;
     {
@@ -574,41 +513,36 @@ hipError_t launch_tiles(const void* A, const void* B, float* C, int M, int N, in
     }
     Schedule sc;
     int grid = 0;
-    if (!make_schedule<WM>(M, N, K, d->slots, d->cus, ws.max_partials, sc, grid)) return hipErrorInvalidValue;
+    if (!make_schedule(M, N, K, d->slots, d->cus, ws.max_partials, sc, grid)) return hipErrorInvalidValue;
     const int nb_k = K / 64;
-    if (WM == 2)
-        hipLaunchKernelGGL(gemm_a81w41_tile64_kernel, dim3(grid), dim3(kTileThreads), Geom<2>::kLdsBytes, s,
-                           static_cast<const uint8_t*>(A), static_cast<const uint8_t*>(B), M, N, nb_k, sc.tiles_m,
-                           sc.tiles_n, sc.whole, sc.r, sc.c, sc.chunk, sc.band, C, ws.partials, ws.arrivals);
-    else {
-        hipLaunchKernelGGL(gemm_a81w41_tile32x128_kernel, dim3(grid), dim3(kTileThreads), Geom<1>::kLdsBytes, s,
-                           static_cast<const uint8_t*>(A), static_cast<const uint8_t*>(B), M, N, nb_k, sc.tiles_m,
-                           sc.tiles_n, sc.whole, sc.r, sc.c, sc.chunk, sc.band, C, ws.partials, ws.arrivals);
-    }
+    hipLaunchKernelGGL(gemm_a81w41_tile64_kernel, dim3(grid), dim3(kTileThreads), Geom::kLdsBytes, s,
+                       static_cast<const uint8_t*>(A), static_cast<const uint8_t*>(B), M, N, nb_k, sc.tiles_m, sc.tiles_n, sc.whole,
+                       sc.r, sc.c, sc.chunk, sc.band, C, ws.partials, ws.arrivals);
     return hipGetLastError();
 }
 
-// Which kernel a call goes to: 0 the few-row kernel (no scratch), 1 the 32 x 128 tiles, 2 the 64 x 64 tiles,
-// 3 the one-row-panel kernel that loads its operands straight into registers (9 .. 32 rows).
+// Which kernel a call goes to: 0 the few-row kernel (no scratch), 2 the 64 x 64 tiles, and for 9 .. 32 rows the
+// one-row-panel kernel: 3 with its operands loaded straight into registers, 4 with wave-private LDS stages.
 int pick_kernel(int M, int N, int K) {
-    // Measurement aids (tuning builds): A81W41_GEMM_TUNE=tile keeps few-row calls on the matrix-core kernels,
-    // A81W41_GEMM_TUNE=Tile64 additionally keeps every call on the 64 x 64 arrangement.
+    // Measurement aids (tuning builds): A81W41_GEMM_TUNE=tile keeps few-row calls off the few-row kernel,
+    // A81W41_GEMM_TUNE=Tile64 keeps every call on the 64 x 64 tiles.
     const char* tune_s = tuning_env("A81W41_GEMM_TUNE");
     const char tune = tune_s ? tune_s[0] : '\0';
     const bool tile_only = tune == 't' || tune == 'T';
     if (!tile_only && gemm_rows_fits(M, K)) return 0;
-    // At most 32 rows: 32 x 128 tiles (no wave idles on rows that do not exist).  Measured at M = 9..32 with
-    // the four-per-CU kernels: N = 12288 17 us against 22 us with 64 x 64 tiles, down_proj (N = 4096,
-    // K = 12288) 21.2 against 24.5, N = 4096 and 1024 at K = 4096 equal.
-    const int env_n = tuning_env_int("A81W41_GEMM_N32X128");
-    const int min_n_32x128 = env_n > 0 ? env_n : 1024;
-    // Narrow layers at 9 .. 32 rows: too few 32 x 128 tiles to go round, so the tile kernels cut K 12- to 16-fold
-    // and the last arriver's merge dominates; the one-row-panel kernel cuts K inside the workgroup instead
-    // (N = 1024, K = 4096: 9.6 against 14.1 us per forward).  From N = 4096 on its per-lane loads of the 80 B
-    // row blocks cost more than the tile kernels' staged copies (gate_proj at 32 rows 32 against 22 us).
-    const int rows32_mode = tuning_env_int("A81W41_GEMM_ROWS32");  // tuning builds: 1 always, 2 never
-    if (M <= 32 && tune != 'T' && rows32_mode != 2 && (N <= 2048 || rows32_mode == 1)) return 3;
-    if (M <= 32 && N >= min_n_32x128 && tune != 'T') return 1;
+    if (M > 32 || tune == 'T') return 2;
+    // At most 32 rows: such a call is bound by streaming the weights once, and 64 x 64 tiles (or 32 x 128 ones, an
+    // arrangement this file used to have) cut K 8- to 16-fold between workgroups, whose last arriver's merge then
+    // dominates; the one-row-panel kernel cuts K inside the workgroup.  Forward at 9 .. 32 rows, us, against the
+    // 32 x 128 tiles: N = 1024, K = 4096 8.9 against 14.1 (registers; staged 9.3); gate_proj 18.0 .. 18.6 against
+    // 20.2 .. 21.5 and down_proj 17.9 .. 18.3 against 22.9 .. 23.2 (staged; with register loads gate_proj at 32 rows
+    // took 32: nine load instructions per wave and super-block on the CU's cache path).
+    const int rows32_mode = tuning_env_int("A81W41_GEMM_ROWS32");         // tuning builds: 1 always registers, 2 never
+    const int staged_mode = tuning_env_int("A81W41_GEMM_ROWS32_STAGED");  // tuning builds: 1 always staged, 2 never
+    if (staged_mode == 1) return 4;
+    if (rows32_mode == 1) return 3;
+    if (N <= 2048 && rows32_mode != 2) return 3;
+    if (staged_mode != 2) return 4;
     return 2;
 }
 
@@ -619,11 +553,13 @@ using namespace gemm_detail;
 const char* gemm_kernel_name(int M, int N, int K) {
     switch (pick_kernel(M, N, K)) {
         case 0: return "rows (2..8 rows resident in LDS, v_dot4, weights streamed once)";
-        case 1: return "tile32x128 (int8 matrix ops, 4 waves side by side, K split)";
         case 3: return "rows32 (int8 matrix ops, one row panel, K split inside the workgroup)";
+        case 4: return "rows32_staged (int8 matrix ops, one row panel, K split inside the workgroup, wave-private LDS stages)";
         default: return "tile64 (int8 matrix ops, 64 x 64 tiles, LDS-staged)";
     }
 }
+
+bool gemm_rows32_staged_preferred(int M, int N, int K) { return M >= 2 && pick_kernel(M, N, K) == 4; }
 
 hipError_t gemm_scratch_create(GemmScratch* out) {
     out->partials = nullptr;
@@ -722,8 +658,8 @@ int gemm_static_scratch_tiles() { return kStaticPartials; }
 int gemm_partial_tiles(int M, int N, int K) {
     const int kernel = pick_kernel(M, N, K);
     if (kernel == 0) return 0;
-    if (kernel == 3) {  // a share of a column panel parks 4 KiB, a quarter of a partial-tile unit
-        const int split = gemm_rows32_split(N, K);
+    if (kernel == 3 || kernel == 4) {  // a share of a column panel parks 4 KiB, a quarter of a partial-tile unit
+        const int split = gemm_rows32_split(N, K, kernel == 4);
         return split > 1 ? ((N + 31) / 32 * split + 3) / 4 : 0;
     }
     std::lock_guard<std::mutex> lock(g_dev_mutex);
@@ -731,10 +667,7 @@ int gemm_partial_tiles(int M, int N, int K) {
     if (device_info_locked(d) != hipSuccess) return -1;
     Schedule sc;
     int grid = 0;
-    if (kernel == 1)
-        make_schedule<1>(M, N, K, d->slots, d->cus, kMaxPartials, sc, grid);
-    else
-        make_schedule<2>(M, N, K, d->slots, d->cus, kMaxPartials, sc, grid);
+    make_schedule(M, N, K, d->slots, d->cus, kMaxPartials, sc, grid);
     return sc.r * sc.c;
 }
 
@@ -747,20 +680,18 @@ hipError_t clear_gemm_counters(const GemmScratch& ws, hipStream_t s) {
 hipError_t launch_gemm_fp32(const void* A, const void* B, float* C, int M, int N, int K, const GemmScratch& ws, hipStream_t s) {
     switch (pick_kernel(M, N, K)) {
         case 0: return launch_gemm_rows_fp32(A, B, C, M, N, K, s);
-        case 1: return launch_tiles<1>(A, B, C, M, N, K, ws, s);
         case 3: return launch_gemm_rows32_fp32(A, B, C, M, N, K, ws, s);
-        default: return launch_tiles<2>(A, B, C, M, N, K, ws, s);
+        case 4: return launch_gemm_rows32_fp32(A, B, C, M, N, K, ws, s, true);
+        default: return launch_tiles(A, B, C, M, N, K, ws, s);
     }
 }
 
 // Host-side check of the work list a launch would walk (no device needed): every whole tile once, every
 // chunk of every split tile once, partial-tile indices distinct and below the scratch size.
-int gemm_schedule_selfcheck(int M, int N, int K, int slots_fit, int cus, int wm) {
+int gemm_schedule_selfcheck(int M, int N, int K, int slots_fit, int cus) {
     Schedule sc;
     int grid = 0;
-    const bool fits = wm == 1 ? make_schedule<1>(M, N, K, slots_fit, cus, kMaxPartials, sc, grid)
-                              : make_schedule<2>(M, N, K, slots_fit, cus, kMaxPartials, sc, grid);
-    if (!fits) return -1;
+    if (!make_schedule(M, N, K, slots_fit, cus, kMaxPartials, sc, grid)) return -1;
     const int T = sc.tiles_m * sc.tiles_n, nb_k = K / 64;
     if (sc.whole + sc.r != T || sc.items != sc.whole + sc.r * sc.c || sc.chunk * sc.c != nb_k) return -2;
     if (grid < 1 || grid > slots_fit) return -3;

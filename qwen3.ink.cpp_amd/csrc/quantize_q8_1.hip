@@ -12,10 +12,13 @@
 namespace a81w41 {
 namespace {
 
+// yt (fp32 parameters only, may be null): a second copy of the blocks with the rows of a super-block next to each
+// other, block (row, sb) at (32 sb + row) * 80 -- what the 9..32-row contraction kernel stages per super-block in
+// one contiguous piece.  nb_k = super-blocks per row; at most 32 rows.
 template <bool FP32, bool ALIGNED>
 __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const float* __restrict__ x,
                                                             uint8_t* __restrict__ y, int64_t nb64,
-                                                            bool write_sums) {
+                                                            bool write_sums, uint8_t* __restrict__ yt, int nb_k) {
     const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;  // one float4 each
     const int64_t sb = t >> 4;
     const int h = (int)(t >> 3) & 1;  // low / high 32-block
@@ -36,6 +39,16 @@ __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const float* __restr
     constexpr int QOFF = FP32 ? 16 : 8;
     uint8_t* blk = y + sb * BS;
     *reinterpret_cast<uint32_t*>(blk + QOFF + 32 * h + 4 * j) = qz.packed;
+    if (FP32 && yt != nullptr) {
+        const int64_t row = sb / nb_k, sbr = sb - row * nb_k;
+        uint8_t* tb = yt + (sbr * 32 + row) * BS;
+        *reinterpret_cast<uint32_t*>(tb + QOFF + 32 * h + 4 * j) = qz.packed;
+        if (j == 0) {
+            float* p = reinterpret_cast<float*>(tb);
+            p[h] = qz.d;
+            p[2 + h] = qz.ssum;
+        }
+    }
     if (j == 0) {
         if (FP32) {
             float* p = reinterpret_cast<float*>(blk);
@@ -51,13 +64,16 @@ __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const float* __restr
 
 }  // namespace
 
-hipError_t launch_quantize(const float* x, void* y, int64_t nb64, bool fp32, hipStream_t s, bool write_sums) {
+hipError_t launch_quantize(const float* x, void* y, int64_t nb64, bool fp32, hipStream_t s, bool write_sums, void* y_by_superblock,
+                           int nb_k) {
     if (nb64 == 0) return hipSuccess;
+    if (y_by_superblock != nullptr && (!fp32 || !write_sums || nb_k < 1 || nb64 % nb_k || nb64 / nb_k > 32)) return hipErrorInvalidValue;
+    uint8_t* yt = static_cast<uint8_t*>(y_by_superblock);
     const int64_t threads = nb64 * 16;
     const unsigned grid = (unsigned)((threads + 255) / 256);
     const bool aligned = (reinterpret_cast<uintptr_t>(x) & 15) == 0;
     uint8_t* yb = static_cast<uint8_t*>(y);
-#define LAUNCH(F, A) hipLaunchKernelGGL((quantize_q8_1_kernel<F, A>), dim3(grid), dim3(256), 0, s, x, yb, nb64, write_sums)
+#define LAUNCH(F, A) hipLaunchKernelGGL((quantize_q8_1_kernel<F, A>), dim3(grid), dim3(256), 0, s, x, yb, nb64, write_sums, yt, nb_k)
     if (fp32) {
         if (aligned) LAUNCH(true, true); else LAUNCH(true, false);
     } else {

@@ -72,25 +72,24 @@ def test_no_gpu_is_reported_not_faked(pkg):
     assert L.a81w41_gemv_repack_A81W41_fp16(p, p, p, 1, 8, 64, None) == 4
 
 
-@pytest.mark.parametrize("tile", [1, 2])
-def test_gemm_schedule_covers_every_tile_and_chunk_once(pkg, tile):
-    """The work list of the M > 8 kernels (persistent grid, last round cut along K): walked on the host for
+def test_gemm_schedule_covers_every_tile_and_chunk_once(pkg):
+    """The work list of the 64 x 64-tile kernel (persistent grid, last round cut along K): walked on the host for
     the shapes and row counts the layer sees and for odd ones, on the real chip size and on smaller ones.
     Every tile and every K chunk exactly once, tile numbering one-to-one, no partial tile shared."""
     L = pkg.capi.lib()
     shapes = [(4096, 4096), (4096, 1024), (4096, 12288), (12288, 4096), (4096, 6144), (4096, 24576),
               (512, 256), (4096, 8), (256, 4104), (64, 64), (1024, 40)]
-    rows = [9, 16, 31, 32] if tile == 1 else [9, 33, 64, 65, 128, 322, 512, 640, 832, 1024, 2048, 4096]
+    rows = [9, 33, 64, 65, 128, 322, 512, 640, 832, 1024, 2048, 4096]
     used_split = 0
     for K, N in shapes:
         for M in rows:
             for resident, cus in ((1024, 256), (512, 256), (768, 256), (16, 4), (3, 3)):
-                got = L.a81w41_gemm_schedule_selfcheck(M, N, K, resident, cus, tile)
-                assert got >= 0, (M, N, K, resident, cus, tile, got)
+                got = L.a81w41_gemm_schedule_selfcheck(M, N, K, resident, cus)
+                assert got >= 0, (M, N, K, resident, cus, got)
                 assert got <= 4096
                 used_split += got > 0
     assert used_split > 20      # the K split really is exercised
-    assert L.a81w41_gemm_schedule_selfcheck(0, 64, 64, 1024, 256, 2) < 0   # argument errors are negative too
+    assert L.a81w41_gemm_schedule_selfcheck(0, 64, 64, 1024, 256) < 0   # argument errors are negative too
 
 
 def test_block_scaled_gemm_plan_covers_every_unit_once(pkg):

@@ -166,11 +166,11 @@ def test_gemv_extreme_codes(pkg, ora, torch):
                                    (322, 96, 1024), (45, 32, 12288), (130, 136, 2048), (70, 520, 64),
                                    (65, 8, 128), (3, 16, 1088), (5, 4096, 4096), (8, 64, 12288), (4, 136, 12288),
                                    (8, 1024, 4096), (9, 64, 12288),
-                                   # 9..32 rows: 64 x 64 tiles for layers under 1024 wide ...
+                                   # 9..32 rows on narrow layers: the one-row-panel kernel with register loads ...
                                    (9, 8, 64), (17, 136, 256), (32, 128, 4096), (31, 1000, 2048), (12, 4096, 4096),
                                    (32, 1024, 12288),
-                                   # ... and the 32 x 128 arrangement from N = 1024 on: ragged N, K not a multiple of
-                                   # the ring, split K, more tiles than workgroup slots
+                                   # ... and with wave-private LDS stages on wide ones: ragged N, K not a multiple of
+                                   # the ring or of the waves, shared K, more panels than workgroup slots
                                    (9, 8200, 64), (17, 9000, 320), (32, 8192, 1024), (20, 72000, 256), (25, 12288, 4096), (21, 1032, 320),
                                    # more tiles than workgroup slots (768): whole rounds plus a K-split partial
                                    # round, ragged rows and columns; 513..682 tiles: the two-per-CU schedule
@@ -527,3 +527,28 @@ def test_few_row_forward_quantises_in_its_prologue(pkg, ora, synth, torch, M, N,
     assert row_err(got.cpu().numpy(), want) <= 5e-6
     # the same kernel without the prologue, on the quantised rows (the free-standing entry point)
     assert torch.equal(got, pkg.ops.gemm_fp32(dev(torch, ba), dev(torch, bw), M, N, K))
+
+
+@pytest.mark.parametrize("N,K", [(4096, 4096), (12288, 4096), (4096, 12288), (4104, 4096), (2056, 320), (6144, 192)])
+def test_9_to_32_rows_on_wide_layers_stage_their_rows_per_super_block(pkg, ora, synth, torch, N, K):
+    """9 .. 32 rows on a layer wider than 2048 columns: the layer's quantiser launch also writes the 80 B blocks with
+    the rows of a super-block next to each other, and the one-row-panel kernel stages them from there.  The scratch
+    holds the oracle's blocks; the output has the bits of the free-standing entry point on those blocks (same
+    kernel, rows staged from the reference's layout) and is within the bar; a call with fewer rows after one with
+    more is not disturbed by the row slots the earlier call left behind."""
+    w4, s, o = synth.weight_files(N, K, 661)
+    s = s * np.float32(0.9371)
+    bw = ora.repack(w4, s, o, K, N, True)
+    ctx = pkg.ops.Context(max_rows=32, max_cols=K)
+    layer = pkg.Linear.from_blobs(None, bw, N, K, ctx)
+    for M in (32, 9, 17, 31):
+        x = synth.activations(M, K, 662 + M, outliers=True)
+        x[M - 1, 64:128] = 0.0                      # an all-zero block: d = 0, id = 0
+        assert layer.kernel_name(M).startswith("rows32_staged")
+        got = layer.forward(dev(torch, x))
+        ba = ora.quantize(x, True)
+        assert np.array_equal(ctx.activation_scratch(M * K // 64 * 80).cpu().numpy(), ba), M
+        want = ora.gemm_fp32(ba, bw, M, N, K)
+        assert row_err(got.cpu().numpy(), want) <= 5e-6, M
+        assert torch.equal(got, pkg.ops.gemm_fp32(dev(torch, ba), dev(torch, bw), M, N, K)), M
+        assert torch.equal(got, layer.forward(dev(torch, x))), M

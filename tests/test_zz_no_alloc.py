@@ -58,8 +58,8 @@ def test_static_scratch_gemm_equals_the_allocating_entry_point(pkg, ora, synth):
     # two calls in a row, the second smaller; then a shape without a K split and a few-row call.
     # (322, 1024, 4096) and (130, 136, 2048) split K (partial tiles parked in the static array).
     cases = [(322, 1024, 4096, 401), (130, 136, 2048, 403), (64, 64, 1024, 405), (5, 64, 256, 407), (322, 1024, 4096, 401)]
-    assert L.a81w41_gemm_schedule_selfcheck(322, 1024, 4096, 1024, 256, 2) > 0
-    assert L.a81w41_gemm_schedule_selfcheck(130, 136, 2048, 1024, 256, 2) > 0
+    assert L.a81w41_gemm_schedule_selfcheck(322, 1024, 4096, 1024, 256) > 0
+    assert L.a81w41_gemm_schedule_selfcheck(130, 136, 2048, 1024, 256) > 0
     for M, N, K, seed in cases:
         a, b, want = _case(ora, synth, torch, M, N, K, seed)
         ref = pkg.ops.gemm_fp32(a, b, M, N, K)
@@ -80,7 +80,7 @@ def test_static_scratch_gemm_rejects_what_does_not_fit(pkg):
     # 700 rows, 704 tiles over K = 12288 cut in four = 2816 > 2048)
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     N, K = 4096, 12288
-    M = next((m for m in range(256, 4096, 4) if L.a81w41_gemm_schedule_selfcheck(m, N, K, 4 * cus, cus, 2) > 2048), None)
+    M = next((m for m in range(256, 4096, 4) if L.a81w41_gemm_schedule_selfcheck(m, N, K, 4 * cus, cus) > 2048), None)
     assert M is not None, "no shape on this device exceeds the static scratch"
     a = torch.zeros(M * (K // 64) * 80, dtype=torch.uint8, device="cuda")
     b = torch.zeros((N // 8) * (K // 64) * 384, dtype=torch.uint8, device="cuda")
