@@ -529,7 +529,10 @@ int pick_kernel(int M, int N, int K) {
     const char* tune_s = tuning_env("A81W41_GEMM_TUNE");
     const char tune = tune_s ? tune_s[0] : '\0';
     const bool tile_only = tune == 't' || tune == 'T';
-    if (!tile_only && gemm_rows_fits(M, K)) return 0;
+    // 7 and 8 rows over a long K on a wide layer: the few-row kernel's time grows by 1.4 us per row there (down_proj:
+    // 19.3 and 20.7 us forward) and passes the one-row-panel kernel's 18 us
+    const bool long_k_rows = M >= 7 && K >= 8192 && N > 2048;
+    if (!tile_only && gemm_rows_fits(M, K) && !long_k_rows) return 0;
     if (M > 32 || tune == 'T') return 2;
     // At most 32 rows: such a call is bound by streaming the weights once, and 64 x 64 tiles (or 32 x 128 ones, an
     // arrangement this file used to have) cut K 8- to 16-fold between workgroups, whose last arriver's merge then

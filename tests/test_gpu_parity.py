@@ -171,7 +171,7 @@ def test_gemv_extreme_codes(pkg, ora, torch):
                                    (32, 1024, 12288),
                                    # ... and with wave-private LDS stages on wide ones: ragged N, K not a multiple of
                                    # the ring or of the waves, shared K, more panels than workgroup slots
-                                   (9, 8200, 64), (17, 9000, 320), (32, 8192, 1024), (20, 72000, 256), (25, 12288, 4096), (21, 1032, 320),
+                                   (8, 4096, 12288), (7, 2056, 8192), (9, 8200, 64), (17, 9000, 320), (32, 8192, 1024), (20, 72000, 256), (25, 12288, 4096), (21, 1032, 320),
                                    # more tiles than workgroup slots (768): whole rounds plus a K-split partial
                                    # round, ragged rows and columns; 513..682 tiles: the two-per-CU schedule
                                    (256, 16384, 256), (322, 12288, 256), (1030, 4104, 256), (384, 24576, 512), (640, 4096, 256)])
