@@ -166,6 +166,8 @@ __global__ __launch_bounds__(kThreads) void gemm_a81w41_rows32_kernel(const uint
             if (c < 160) {
                 const int rw = c / 5, piece = c - 5 * rw;
                 if (At != nullptr) {  // the rows of a super-block next to each other: 2560 contiguous bytes per stage
+                    // (row slots past M hold whatever an earlier call left there: a row's values only ever reach
+                    // that row's outputs, which are not stored)
                     cp.src[i] = At + ((size_t)k_lo * 32 + rw) * kABlock32 + 16 * piece;
                     cp.step[i] = 32 * kABlock32;
                 } else {
